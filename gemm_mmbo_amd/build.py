@@ -1,0 +1,82 @@
+"""Build libmmbo_gemm.so (the C-ABI library with every gfx950 kernel) in-tree with hipcc.
+
+    python -m gemm_mmbo_amd.build [--force]
+
+Each (element type, tile row) pair is its own translation unit so the kernels compile in
+parallel; objects go to gemm_mmbo_amd/csrc/build/, the library to gemm_mmbo_amd/csrc/.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(CSRC, "libmmbo_gemm.so")
+
+NUM_TILES = 6  # keep in step with csrc/configs.hpp
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # no packed-fp32 VALU forms: some of them have produced wrong results on this hardware
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _units():
+    units = [("mmbo_gemm.hip", "mmbo_gemm.o", [])]
+    for dtype in (0, 1):
+        for tile in range(NUM_TILES):
+            units.append(("inst_staged.hip", f"inst_staged_{dtype}_{tile}.o",
+                          [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
+    extra = os.path.join(CSRC, "extra_units.txt")
+    if os.path.exists(extra):
+        for line in open(extra):
+            line = line.split("#")[0].split()
+            if line:
+                units.append((line[0], line[1], line[2:]))
+    return units
+
+
+def _deps():
+    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".hip", ".txt"))] + \
+           [os.path.join(HERE, "..", "include", "mmbo_gemm.h")]
+
+
+def _compile(unit, force, newest_dep):
+    src, obj, defs = unit
+    objp = os.path.join(OBJ, obj)
+    if not force and os.path.exists(objp) and os.path.getmtime(objp) >= newest_dep:
+        return obj, "up to date"
+    cmd = [HIPCC] + FLAGS + defs + ["-c", os.path.join(CSRC, src), "-o", objp]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {obj}:\n{' '.join(cmd)}\n{r.stderr[-4000:]}")
+    return obj, "compiled"
+
+
+def build(force=False, verbose=True, jobs=None):
+    os.makedirs(OBJ, exist_ok=True)
+    newest = max(os.path.getmtime(p) for p in _deps())
+    units = _units()
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(lambda u: _compile(u, force, newest), units))
+    if verbose:
+        for obj, what in results:
+            print(f"  {obj}: {what}")
+    objs = [os.path.join(OBJ, u[1]) for u in units]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    if verbose:
+        print(f"  linked {LIB}")
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

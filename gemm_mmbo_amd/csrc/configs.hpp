@@ -1,0 +1,39 @@
+// Tile-config table: the successor of the reference's {MT0I, MT1J, threads} rows
+// (src/gemm/constants.h:34-47,106-135), retuned for 256 CUs, 64-wide wavefronts and 32x32 MFMA blocks.
+//
+// A config id is  tile + NUM_TILES * split_index : every tile shape can run with
+// GlobalSplitU = 1, 2, 4, 8 or 16 (the reference's kernels are all GSU01).
+#pragma once
+
+namespace mmbo {
+
+struct TileRow {
+    int bm, bn, bk;   // macro tile MT0I x MT1J x DepthU
+    int wm, wn;       // wavefronts along M and N; wave tile = (bm/wm) x (bn/wn)
+};
+
+constexpr int NUM_TILES = 6;
+constexpr int NUM_SPLITS = 5;
+constexpr int kSplits[NUM_SPLITS] = {1, 2, 4, 8, 16};
+
+//                                              bm   bn  bk wm wn
+constexpr TileRow kTilesF32[NUM_TILES] = {
+    {256, 256, 16, 2, 4},
+    {256, 128, 16, 2, 2},
+    {128, 128, 16, 2, 2},
+    {128,  64, 16, 2, 2},
+    { 64,  64, 32, 2, 2},
+    { 32,  32, 32, 1, 1},
+};
+constexpr TileRow kTilesF16[NUM_TILES] = {
+    {256, 256, 64, 2, 4},
+    {256, 128, 64, 2, 2},
+    {128, 128, 64, 2, 2},
+    {128,  64, 64, 2, 2},
+    { 64,  64, 64, 2, 2},
+    { 32,  32, 64, 1, 1},
+};
+
+constexpr const TileRow &tile_row(int dtype, int tile) { return dtype == 0 ? kTilesF32[tile] : kTilesF16[tile]; }
+
+}  // namespace mmbo

@@ -1,0 +1,87 @@
+// Shared device/host definitions for the gfx950 GEMM kernels.
+//
+// Index convention (reference: src/gemm/ref/Kernels.cpp:76-78): i runs over M, j over N, l over K,
+// and the grid's z over the batch; all storage is column-major.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mmbo {
+
+typedef _Float16 half_t;
+typedef float    f32x4  __attribute__((ext_vector_type(4)));
+typedef float    f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8  __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4  __attribute__((ext_vector_type(4)));
+typedef short    i16x4  __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4  __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2  __attribute__((ext_vector_type(2)));
+
+#define MMBO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// Kernel argument block.  Successor of the reference's packed kernarg structs
+// (src/gemm/gemm.h:6-23 and :49-72): same fields -- C/A/B, alpha/beta, the three leading
+// dimensions, sizeI/J/L, the batch strides -- plus what split-K and the tile mapping need.
+struct GemmArgs {
+    const void *A;
+    const void *B;
+    void *C;
+    float *ws;              // split-K partial sums: [split][batch][n][m] fp32, dense
+    float alpha;
+    float beta;
+    uint32_t m, n, k;       // sizeI, sizeJ, sizeL
+    uint32_t lda, ldb, ldc; // strideA1L/strideB1L/strideC1J, in elements
+    int64_t strideA, strideB, strideC;   // batch strides in elements (strideA2K/B2K/C2K)
+    uint32_t nwg0, nwg1;    // tiles along M and N
+    uint32_t wgm;           // WorkGroupMapping width (reference: 8)
+    uint32_t nxcd;          // XCDs the dispatcher round-robins over (8 on MI355X; 1 = plain order)
+    uint32_t splits;        // GlobalSplitU
+    uint32_t k_per_split;   // multiple of the config's depthU
+    uint32_t batch;
+    uint32_t vec_a, vec_b, vec_c;   // 1 when 128-bit accesses to that operand are aligned
+};
+
+// Linear work-group id -> (tile row, tile column).
+//
+// Step 1 (nxcd > 1): hardware hands consecutive ids to XCDs round-robin, each XCD with its own L2.
+// Regroup so XCD x gets the contiguous run of ids [start_x, start_x + count_x): neighbours in the
+// remapped order then share an L2.
+// Step 2: the reference's WorkGroupMapping (src/gemm/ref/Kernels.cpp:204-236): walk `wgm` tile
+// columns wide, down all tile rows, then the next block of columns; the trailing block is as wide
+// as what is left.  With nxcd == 1 and id = wg0 + wg1*nwg0 this is that remap exactly.
+__host__ __device__ inline void wg_remap(uint32_t id, uint32_t nwg0, uint32_t nwg1, uint32_t wgm,
+                                         uint32_t nxcd, uint32_t &wg0, uint32_t &wg1)
+{
+    uint32_t total = nwg0 * nwg1;
+    if (nxcd > 1 && total >= nxcd) {
+        uint32_t per = (total + nxcd - 1) / nxcd;        // ids on the fuller XCDs
+        uint32_t tall = total % nxcd == 0 ? nxcd : total % nxcd;
+        uint32_t x = id % nxcd, local = id / nxcd;
+        id = x < tall ? x * per + local : tall * per + (x - tall) * (per - 1) + local;
+    }
+    uint32_t g0 = id % nwg0, g1 = id / nwg0;
+    if (wgm <= 1) { wg0 = g0; wg1 = g1; return; }
+    uint32_t serial = g0 + (g1 % wgm) * nwg0;
+    uint32_t block = g1 / wgm;
+    uint32_t rem = (g1 < nwg1 - (nwg1 % wgm)) ? 0u : nwg1 % wgm;
+    uint32_t width = rem == 0 ? wgm : rem;
+    wg0 = serial / width;
+    wg1 = serial % width + block * wgm;
+}
+
+template <typename T> struct ElemTraits;
+template <> struct ElemTraits<float> {
+    static constexpr int VEC = 4;      // elements per 128-bit access
+    static constexpr int KG = 8;       // k extent covered by one round of LDS fragment reads
+    static constexpr int PAD_KC = 4;   // row padding (elements) of a k-contiguous LDS tile: 16 B
+    static constexpr int PAD_RC = 8;   // row padding of a row-contiguous LDS tile
+};
+template <> struct ElemTraits<half_t> {
+    static constexpr int VEC = 8;
+    static constexpr int KG = 16;
+    static constexpr int PAD_KC = 8;   // 16 B
+    static constexpr int PAD_RC = 32;  // 64 B: the four k-rows of one transposed read land in distinct bank groups
+};
+
+}  // namespace mmbo

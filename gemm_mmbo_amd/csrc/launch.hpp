@@ -1,0 +1,20 @@
+// Launchers: one explicit specialisation per (element type, tile row), each defined in its own
+// translation unit (inst_staged.hip compiled once per pair) so the kernels build in parallel.
+#pragma once
+
+#include "gemm_common.hpp"
+
+namespace mmbo {
+
+// dtype: 0 = fp32, 1 = fp16.  Launches the staged kernel for tile row TILE with the given
+// transposes; grid = (nwg0*nwg1, 1, batch*splits).  Returns the launch's hipError_t.
+template <int DTYPE, int TILE>
+hipError_t launch_staged(int transA, int transB, const GemmArgs &args, hipStream_t stream);
+
+// LDS bytes the staged kernel of that tile needs, worst case over the four transposes.
+template <int DTYPE, int TILE>
+int staged_lds_bytes();
+
+hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream);
+
+}  // namespace mmbo

@@ -1,0 +1,330 @@
+// C ABI of the gfx950 GEMM library: argument checking, tile-config table, per-shape selection,
+// split-K workspace and kernel dispatch.  The reference's counterpart is the header-inline host
+// layer src/gemm/gemm.h (front-ends), src/gemm/constants.h (tables) and src/gemm/driver.h (launch).
+#include "../../include/mmbo_gemm.h"
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "configs.hpp"
+#include "gemm_common.hpp"
+#include "gemm_staged.hpp"
+#include "launch.hpp"
+
+namespace mmbo {
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+int hip_fail(hipError_t e)
+{
+    g_last_hip_error = (int)e;
+    return MMBO_ERR_HIP;
+}
+
+// ---- split-K workspace: one grow-only buffer per device ---------------------------------------
+constexpr int kMaxDevices = 64;
+std::mutex g_ws_mutex;
+float *g_ws[kMaxDevices] = {};
+size_t g_ws_bytes[kMaxDevices] = {};
+
+int workspace(size_t bytes, float **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (g_ws_bytes[dev] < bytes) {
+        if (g_ws[dev]) {
+            // earlier launches may still be reading the old buffer
+            e = hipDeviceSynchronize();
+            if (e != hipSuccess) return hip_fail(e);
+            (void)hipFree(g_ws[dev]);
+            g_ws[dev] = nullptr;
+            g_ws_bytes[dev] = 0;
+        }
+        size_t want = bytes + bytes / 4;
+        if (hipMalloc(reinterpret_cast<void **>(&g_ws[dev]), want) != hipSuccess) {
+            (void)hipGetLastError();
+            if (hipMalloc(reinterpret_cast<void **>(&g_ws[dev]), bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                g_ws[dev] = nullptr;
+                return MMBO_ERR_WORKSPACE;
+            }
+            want = bytes;
+        }
+        g_ws_bytes[dev] = want;
+    }
+    *out = g_ws[dev];
+    return MMBO_OK;
+}
+
+// ---- table ------------------------------------------------------------------------------------
+template <int DTYPE, int TILE>
+hipError_t dispatch_tile(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
+{
+    if (tile == TILE) return launch_staged<DTYPE, TILE>(ta, tb, a, s);
+    if constexpr (TILE + 1 < NUM_TILES) return dispatch_tile<DTYPE, TILE + 1>(tile, ta, tb, a, s);
+    return hipErrorInvalidValue;
+}
+
+template <int DTYPE, int TILE>
+int lds_bytes_of(int tile)
+{
+    if (tile == TILE) return staged_lds_bytes<DTYPE, TILE>();
+    if constexpr (TILE + 1 < NUM_TILES) return lds_bytes_of<DTYPE, TILE + 1>(tile);
+    return 0;
+}
+
+inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+
+// Relative cost of one k-step of a tile, per element of C: smaller tiles re-read more of A and B
+// per flop and keep fewer MFMAs in flight.  Hand-set from measurements on MI355X.
+double tile_cost(int dtype, int tile)
+{
+    static const double c32[NUM_TILES] = {1.00, 1.05, 1.15, 1.40, 1.9, 6.0};
+    static const double c16[NUM_TILES] = {1.00, 1.15, 1.35, 1.80, 2.6, 8.0};
+    return dtype == MMBO_F32 ? c32[tile] : c16[tile];
+}
+
+// Modelled time (arbitrary units) of running the problem with (tile, split).
+double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, int batch)
+{
+    const TileRow &r = tile_row(dtype, tile);
+    const double cus = 256.0;
+    double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch * split;
+    // work-groups resident per CU, bounded by LDS (160 KB) and by 2048 threads
+    int lds = dtype == MMBO_F32 ? lds_bytes_of<0, 0>(tile) : lds_bytes_of<1, 0>(tile);
+    int per_cu = 160 * 1024 / (lds > 0 ? lds : 1);
+    int thr = r.wm * r.wn * 64;
+    if (per_cu > 2048 / thr) per_cu = 2048 / thr;
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 4) per_cu = 4;
+    double slots = cus * per_cu;
+    double rounds = (double)ceil_div((size_t)tiles, (size_t)slots);
+    // tiles sharing a CU share its MFMA pipes
+    double conc = tiles < slots ? (tiles > cus ? tiles / cus : 1.0) : per_cu;
+    double ksteps = (double)ceil_div(ceil_div(k, (size_t)split), (size_t)r.bk) * r.bk;
+    double per_tile = (double)r.bm * r.bn * (ksteps + 4.0 * r.bk) * tile_cost(dtype, tile) * conc;
+    double t = rounds * per_tile;
+    if (split > 1) t += (double)m * n * batch * (split + 2) * 64.0 / cus;   // partial-sum write + reduce pass
+    return t;
+}
+
+}  // namespace
+
+hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream)
+{
+    size_t mn = (size_t)args.m * args.n;
+    dim3 grid((unsigned)ceil_div(mn, 256), 1, args.batch);
+    if (dtype == MMBO_F32) hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, stream, args);
+    else hipLaunchKernelGGL(splitk_reduce_kernel<half_t>, grid, dim3(256), 0, stream, args);
+    return hipGetLastError();
+}
+
+}  // namespace mmbo
+
+using namespace mmbo;
+
+extern "C" {
+
+const char *mmbo_version(void) { return "mmbo_gemm 0.1 (gfx950)"; }
+
+int mmbo_last_hip_error(void) { return g_last_hip_error; }
+
+const char *mmbo_status_string(int status)
+{
+    switch (status) {
+        case MMBO_OK: return "ok";
+        case MMBO_ERR_INVALID_DTYPE: return "invalid dtype";
+        case MMBO_ERR_INVALID_OP: return "invalid transpose op";
+        case MMBO_ERR_INVALID_SIZE: return "invalid size, leading dimension, stride or batch";
+        case MMBO_ERR_NULL_POINTER: return "null pointer";
+        case MMBO_ERR_INVALID_CONFIG: return "invalid config id";
+        case MMBO_ERR_HIP: return "HIP runtime error";
+        case MMBO_ERR_NO_DEVICE: return "no usable device";
+        case MMBO_ERR_WORKSPACE: return "split-K workspace allocation failed";
+        default: return "unknown status";
+    }
+}
+
+int mmbo_num_configs(int dtype)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
+    return NUM_TILES * NUM_SPLITS;
+}
+
+int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if (!out) return MMBO_ERR_NULL_POINTER;
+    if (config_id < 0 || config_id >= NUM_TILES * NUM_SPLITS) return MMBO_ERR_INVALID_CONFIG;
+    int tile = config_id % NUM_TILES, split = kSplits[config_id / NUM_TILES];
+    const TileRow &r = tile_row(dtype, tile);
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d", r.bm, r.bn, r.bk,
+                  r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, split);
+    out->macro_tile_m = r.bm;
+    out->macro_tile_n = r.bn;
+    out->depth_u = r.bk;
+    out->threads = r.wm * r.wn * 64;
+    out->wave_tile_m = r.bm / r.wm;
+    out->wave_tile_n = r.bn / r.wn;
+    out->split_k = split;
+    out->lds_bytes = dtype == MMBO_F32 ? lds_bytes_of<0, 0>(tile) : lds_bytes_of<1, 0>(tile);
+    return MMBO_OK;
+}
+
+int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
+    if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
+    if (batch < 0) return -MMBO_ERR_INVALID_SIZE;
+    if (m == 0 || n == 0 || batch == 0) return 0;
+    int best = 0;
+    double best_t = 0.0;
+    for (int si = 0; si < NUM_SPLITS; ++si) {
+        int split = kSplits[si];
+        for (int tile = 0; tile < NUM_TILES; ++tile) {
+            const TileRow &r = tile_row(dtype, tile);
+            if (split > 1 && ceil_div(k, (size_t)split) < (size_t)2 * r.bk) continue;   // slices too thin
+            double t = model_time(dtype, tile, split, m, n, k ? k : 1, batch);
+            if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
+        }
+    }
+    return best;
+}
+
+int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
+                  unsigned *wg0, unsigned *wg1)
+{
+    if (!wg0 || !wg1) return MMBO_ERR_NULL_POINTER;
+    if (nwg0 == 0 || nwg1 == 0 || wgm == 0 || num_xcd == 0) return MMBO_ERR_INVALID_SIZE;
+    if ((unsigned long long)nwg0 * nwg1 > 0xFFFFFFFFull || linear_id >= nwg0 * nwg1) return MMBO_ERR_INVALID_SIZE;
+    uint32_t a, b;
+    wg_remap(linear_id, nwg0, nwg1, wgm, num_xcd, a, b);
+    *wg0 = a;
+    *wg1 = b;
+    return MMBO_OK;
+}
+
+int mmbo_release_workspace(void)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (g_ws[dev]) {
+        e = hipDeviceSynchronize();
+        if (e != hipSuccess) return hip_fail(e);
+        e = hipFree(g_ws[dev]);
+        g_ws[dev] = nullptr;
+        g_ws_bytes[dev] = 0;
+        if (e != hipSuccess) return hip_fail(e);
+    }
+    return MMBO_OK;
+}
+
+int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+                              const void *alpha, const void *A, size_t lda, long long strideA,
+                              const void *B, size_t ldb, long long strideB, const void *beta, void *C,
+                              size_t ldc, long long strideC, int batch, int config_id, void *stream)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if ((transA & ~1) || (transB & ~1)) return MMBO_ERR_INVALID_OP;
+    if (!alpha || !beta) return MMBO_ERR_NULL_POINTER;
+    const size_t kMaxDim = 0x7FFFFFFFull;
+    if (m > kMaxDim || n > kMaxDim || k > kMaxDim || lda > kMaxDim || ldb > kMaxDim || ldc > kMaxDim)
+        return MMBO_ERR_INVALID_SIZE;
+    if (batch < 0 || batch > 65535) return MMBO_ERR_INVALID_SIZE;
+    // BLAS rule: a leading dimension is at least 1 and at least the operand's stored row count
+    {
+        size_t need_a = transA ? k : m, need_b = transB ? n : k;
+        if (lda < (need_a ? need_a : 1) || ldb < (need_b ? need_b : 1) || ldc < (m ? m : 1))
+            return MMBO_ERR_INVALID_SIZE;
+    }
+    if (strideA < 0 || strideB < 0 || strideC < 0) return MMBO_ERR_INVALID_SIZE;
+    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= NUM_TILES * NUM_SPLITS))
+        return MMBO_ERR_INVALID_CONFIG;
+    if (m == 0 || n == 0 || batch == 0) return MMBO_OK;          // nothing to write
+    if (!C) return MMBO_ERR_NULL_POINTER;
+    if (k != 0 && (!A || !B)) return MMBO_ERR_NULL_POINTER;
+
+    const float alpha_f = *static_cast<const float *>(alpha);
+    const float beta_f = *static_cast<const float *>(beta);
+
+    if (config_id == MMBO_CONFIG_AUTO) {
+        config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
+        if (config_id < 0) return -config_id;
+    }
+    int tile = config_id % NUM_TILES;
+    int split = kSplits[config_id / NUM_TILES];
+    const TileRow &r = tile_row(dtype, tile);
+    const size_t esz = dtype == MMBO_F32 ? 4 : 2;
+
+    // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
+    {
+        size_t span_a = (transA ? (size_t)r.bm : (size_t)r.bk) * lda * esz;
+        size_t span_b = (transB ? (size_t)r.bk : (size_t)r.bn) * ldb * esz;
+        if (span_a >= 0x7FFFFF00ull || span_b >= 0x7FFFFF00ull) return MMBO_ERR_INVALID_CONFIG;
+    }
+
+    size_t nwg0 = ceil_div(m, r.bm), nwg1 = ceil_div(n, r.bn);
+    if (nwg0 * nwg1 > 0x7FFFFFFFull) return MMBO_ERR_INVALID_SIZE;
+    // split-K: slices are whole stages; never more slices than stages
+    size_t stages = ceil_div(k, r.bk);
+    if (stages < 1) stages = 1;
+    if ((size_t)split > stages) split = (int)stages;
+    size_t k_per_split = ceil_div(stages, (size_t)split) * r.bk;
+    split = (int)ceil_div(k ? k : 1, k_per_split);
+    if ((size_t)batch * split > 65535) return MMBO_ERR_INVALID_SIZE;
+
+    GemmArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.A = A; a.B = B; a.C = C; a.ws = nullptr;
+    a.alpha = alpha_f; a.beta = beta_f;
+    a.m = (uint32_t)m; a.n = (uint32_t)n; a.k = (uint32_t)k;
+    a.lda = (uint32_t)lda; a.ldb = (uint32_t)ldb; a.ldc = (uint32_t)ldc;
+    a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;
+    a.nwg0 = (uint32_t)nwg0; a.nwg1 = (uint32_t)nwg1;
+    a.wgm = 8;
+    a.nxcd = 8;
+    a.splits = (uint32_t)split;
+    a.k_per_split = (uint32_t)(split > 1 ? k_per_split : (k ? k : 1));
+    a.batch = (uint32_t)batch;
+    auto aligned16 = [&](const void *p, size_t ld, long long stride) {
+        return ((uintptr_t)p % 16 == 0) && ((ld * esz) % 16 == 0) && (((size_t)stride * esz) % 16 == 0);
+    };
+    a.vec_a = aligned16(A, lda, strideA);
+    a.vec_b = aligned16(B, ldb, strideB);
+    a.vec_c = aligned16(C, ldc, strideC);
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (split > 1) {
+        size_t bytes = (size_t)split * batch * m * n * sizeof(float);
+        int rc = workspace(bytes, &a.ws);
+        if (rc != MMBO_OK) return rc;
+    }
+    hipError_t e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(tile, transA, transB, a, s)
+                                     : dispatch_tile<1, 0>(tile, transA, transB, a, s);
+    if (e != hipSuccess) return hip_fail(e);
+    if (split > 1) {
+        e = launch_splitk_reduce(dtype, a, s);
+        if (e != hipSuccess) return hip_fail(e);
+    }
+    return MMBO_OK;
+}
+
+int mmbo_gemm(int dtype, int transA, int transB, size_t m, size_t n, size_t k, const void *alpha,
+              const void *A, size_t lda, const void *B, size_t ldb, const void *beta, void *C, size_t ldc,
+              int config_id, void *stream)
+{
+    return mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc,
+                                     0, 1, config_id, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,117 @@
+/*
+ * mmbo_gemm.h -- C ABI of the MI355X (gfx950) SGEMM/HGEMM library.
+ *
+ * Plain C: pointers, sizes and status codes only.  Every entry point names the piece of
+ * the reference harness (CSWater/GEMM_MMBO, paths relative to its tree) that it replaces.
+ *
+ * Conventions shared by all GEMM entry points (reference: src/gemm/ref/Kernels.cpp:76-78,84-87,
+ * src/gemm/gemm.h:4-5,28-40):
+ *   - column-major storage:  op(A) is m x k, op(B) is k x n, C is m x n;
+ *       transA == N:  A[i + l*lda]      transA == T:  A[l + i*lda]
+ *       transB == N:  B[l + j*ldb]      transB == T:  B[j + l*ldb]
+ *       C[i + j*ldc]
+ *   - C = alpha * op(A) * op(B) + beta * C;  when beta == 0, C is never read
+ *     (it may hold NaN or Inf) -- src/gemm/ref/Kernels.cpp:87;
+ *   - A, B, C are DEVICE pointers owned by the caller (src/gemm/test.cc:53-66);
+ *     alpha and beta are HOST pointers read before the call returns (src/gemm/gemm.h:31-32);
+ *   - MMBO_F32: float A, B, C, alpha, beta; fp32 MFMA accumulate.
+ *     MMBO_F16: IEEE binary16 A, B, C; alpha and beta are float; fp32 MFMA accumulate,
+ *     one round-to-nearest-even to binary16 on the store;
+ *   - the launch is asynchronous on `stream` (a hipStream_t, NULL = the null stream the
+ *     reference uses, src/gemm/common.h:12); the caller synchronises;
+ *   - config_id selects a row of the tile-config table, like the reference's kernelId
+ *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick;
+ *   - errors come back as status codes; nothing calls exit() (the reference's HIP_CHECK
+ *     does, src/gemm/common.h:20-24).
+ */
+#ifndef MMBO_GEMM_H
+#define MMBO_GEMM_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MMBO_F32 0
+#define MMBO_F16 1
+
+#define MMBO_OP_N 0
+#define MMBO_OP_T 1
+
+#define MMBO_CONFIG_AUTO (-1)
+
+typedef enum mmbo_status {
+    MMBO_OK = 0,
+    MMBO_ERR_INVALID_DTYPE = 1,
+    MMBO_ERR_INVALID_OP = 2,
+    MMBO_ERR_INVALID_SIZE = 3,      /* ld too small, negative batch, dimension beyond 2^31-1 */
+    MMBO_ERR_NULL_POINTER = 4,
+    MMBO_ERR_INVALID_CONFIG = 5,    /* config_id outside the table, or not usable for this call */
+    MMBO_ERR_HIP = 6,               /* a HIP runtime call failed; mmbo_last_hip_error() has the code */
+    MMBO_ERR_NO_DEVICE = 7,         /* no gfx950 device is current */
+    MMBO_ERR_WORKSPACE = 8          /* split-K workspace could not be allocated */
+} mmbo_status;
+
+/* One row of the tile-config table (reference: the {MT0I, MT1J, threads} triples of
+ * src/gemm/constants.h:34-47 and the solution dumps of src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml). */
+typedef struct mmbo_config_desc {
+    char name[64];          /* e.g. "MT256x256x64_WT128x064_W8_SK1"                       */
+    int macro_tile_m;       /* MT0I: rows of C per work-group                              */
+    int macro_tile_n;       /* MT1J: columns of C per work-group                           */
+    int depth_u;            /* DepthU: k extent of one LDS stage                           */
+    int threads;            /* work-group size (multiple of 64)                            */
+    int wave_tile_m;        /* rows of C per wavefront (the MFMA-era "thread tile")        */
+    int wave_tile_n;        /* columns of C per wavefront                                  */
+    int split_k;            /* GlobalSplitU: 1 = none; >1 = partial sums + deterministic reduce */
+    int lds_bytes;          /* LDS per work-group, worst case over the four transposes     */
+} mmbo_config_desc;
+
+/* GEMM.  Replaces naive_dgemm() / dgemm_NT() + launchGemm()
+ * (src/gemm/gemm.h:4-45,47-97, src/gemm/driver.h:15-61): same argument meaning and order
+ * (m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId), with the element type and the two
+ * transposes made parameters instead of being baked into the function and kernel names. */
+int mmbo_gemm(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+              const void *alpha, const void *A, size_t lda, const void *B, size_t ldb,
+              const void *beta, void *C, size_t ldc, int config_id, void *stream);
+
+/* Strided-batched GEMM: batch b uses A + b*strideA, B + b*strideB, C + b*strideC (strides in
+ * elements).  The reference has no host API for it, but its kernel ABI carries the batch index
+ * (sizeK, strideA2K/strideB2K/strideC2K in src/gemm/gemm.h:61-69,82-89; wgK = group_id(2) in
+ * src/gemm/ref/Kernels.cpp:254); this is that capability exposed. */
+int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+                              const void *alpha, const void *A, size_t lda, long long strideA,
+                              const void *B, size_t ldb, long long strideB,
+                              const void *beta, void *C, size_t ldc, long long strideC,
+                              int batch, int config_id, void *stream);
+
+/* Tile-config table access.  Replaces indexing the parallel arrays of src/gemm/constants.h
+ * and the NUM_KERNELS sweep bound of src/gemm/benchmark.cc:10,89-109. */
+int mmbo_num_configs(int dtype);
+int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out);
+
+/* The per-shape pick (reference: the exact-size -> solution table of
+ * src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:929-1177).  Returns a config id >= 0, or a
+ * negative mmbo_status on bad arguments.  Pure host logic: needs no device. */
+int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch);
+
+/* Host twin of the kernels' work-group -> tile mapping: linear work-group id to (tile row, tile
+ * column).  With num_xcd = 1 and linear_id = wg0 + wg1*nwg0 this is the reference's
+ * WorkGroupMapping remap (src/gemm/ref/Kernels.cpp:204-236, src/gemm/ref/map.cpp:11-38);
+ * num_xcd = 8 first regroups the round-robin XCD dispatch order so each XCD owns a contiguous
+ * run of ids.  Pure host logic. */
+int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
+                  unsigned *wg0, unsigned *wg1);
+
+/* Release the split-K workspace held for the current device (allocated lazily, grown on
+ * demand, reused across calls).  The reference never frees what it loads (src/gemm/driver.h:41). */
+int mmbo_release_workspace(void);
+
+const char *mmbo_status_string(int status);
+int mmbo_last_hip_error(void);       /* hipError_t of the last MMBO_ERR_HIP on this thread */
+const char *mmbo_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
