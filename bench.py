@@ -1,0 +1,153 @@
+"""Headline benchmark: GEMM TFLOP/s at 8192^3 on one MI355X, fp16 (value) and fp32 (in "also").
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+A step is one GEMM launch through the C ABI on operands already resident in HBM.  Prints ONE JSON line.
+The timed region holds exactly K launches between two stream synchronisations; the per-launch duration
+used for the roofline comes from HIP events recorded on the same stream around the same K launches.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "GEMM TFLOP/s + % of MFMA peak, fp16 & fp32 at 8192^3, 1 MI355X"
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}      # MI355X published dense matrix peaks
+
+
+def time_gemm(G, torch, dtype, m, n, k, steps, warmup, seed):
+    """Returns (wall ms per step, event ms per launch, config name, device tensors)."""
+    tdt = torch.float32 if dtype == G.F32 else torch.float16
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    if dtype == G.F16:      # A, B ~ N(0,1)*0.1 rounded to fp16
+        A = (torch.randn(m * k, device="cuda", generator=gen) * 0.1).to(tdt)
+        B = (torch.randn(k * n, device="cuda", generator=gen) * 0.1).to(tdt)
+    else:                   # A, B ~ U[-1,1]
+        A = torch.rand(m * k, device="cuda", generator=gen) * 2 - 1
+        B = torch.rand(k * n, device="cuda", generator=gen) * 2 - 1
+    C = torch.full((m * n,), float("nan"), device="cuda", dtype=tdt)     # beta = 0: never read
+    stream = torch.cuda.current_stream()
+    cid = G.select_config(dtype, 0, 0, m, n, k, 1)
+
+    def step():
+        G.gemm(dtype, G.OP_N, G.OP_N, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
+    return wall_ms, ev_ms, G.config_info(dtype, cid), (A, B, C)
+
+
+def spot_check(G, dtype, m, n, k, A, B, C):
+    """A band of 64 rows of C against the fp64 oracle (the full check lives in tests/)."""
+    import numpy as np
+    from oracle import oracle as O
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import util as U
+    hA, hB, hC = A.cpu().numpy(), B.cpu().numpy(), C.cpu().numpy()
+    r0 = 4000
+    want = O.gemm_f64(dtype, 0, 0, 64, n, k, 1.0, hA[r0:], m, hB, k, 0.0, None, m)
+    floor = float(np.sqrt(np.mean(want * want)))
+    rel, _ = O.max_rel_err(dtype, hC[r0:], m, want, 64, n, floor=floor)
+    return rel, U.tol(dtype, k), (hA, hB)
+
+
+def cpu_baseline(dtype, m, n, k, hA, hB):
+    """The oracle's native-precision CPU GEMM (fp16 operands widened to fp32, fp32 multiply-add chains) on
+    the same operands, all host cores, whole problem once."""
+    import numpy as np
+    from oracle import oracle as O
+    hC = np.zeros(m * n, dtype=hA.dtype)
+    O.gemm_native(dtype, 0, 0, 256, 256, 256, 1.0, hA, m, hB, k, 0.0, hC, m)       # spin up the thread pool
+    t0 = time.perf_counter()
+    O.gemm_native(dtype, 0, 0, m, n, k, 1.0, hA, m, hB, k, 0.0, hC, m)
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * m * n * k / dt * 1e-12, 4), "unit": "TFLOP/s", "cores": O.num_threads(),
+            "kind": "port", "seconds": round(dt, 2),
+            "sample": f"the whole {m}x{n}x{k} problem once, same operands as the GPU run"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["f16", "f32"], default=None, help="run one leg only (profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this library runs one GEMM on one GPU; --gpus must be 1 "
+              "(sharding over M/N needs no exchange and is not part of this build)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import gemm_mmbo_amd as G
+    G.lib()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    m = n = k = 8192
+    flops = 2.0 * m * n * k
+    out = {}
+    res = {}
+    for name, dtype in (("f16", G.F16), ("f32", G.F32)):
+        if args.only and args.only != name:
+            continue
+        steps = args.steps if name == "f16" else max(3, args.steps // 4)
+        wall_ms, ev_ms, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, args.warmup, seed=1234)
+        rel, limit, host = spot_check(G, dtype, m, n, k, *tensors)
+        res[name] = dict(wall_ms=wall_ms, ev_ms=ev_ms, cfg=cfg, rel=rel, limit=limit, steps=steps)
+        if name == "f16" and not args.no_cpu:
+            res[name]["cpu"] = cpu_baseline(dtype, m, n, k, *host)
+        del tensors, host
+        torch.cuda.empty_cache()
+
+    head = "f16" if "f16" in res else "f32"
+    r = res[head]
+    tflops = flops / r["wall_ms"] * 1e-9
+    achieved = flops / r["ev_ms"] * 1e-9
+    alg_bytes = (m * k + k * n + m * n) * (2 if head == "f16" else 4)
+    out = {
+        "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": r["steps"],
+        "warmup": args.warmup, "ms_per_step": round(r["wall_ms"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head, "data": "synthetic",
+        "config": {"workload": f"{'H' if head == 'f16' else 'S'}GEMM NN M=N=K=8192 lda=ldb=ldc=8192 alpha=1 beta=0, "
+                               + ("A,B ~ N(0,1)*0.1 rounded to fp16, fp32 accumulate" if head == "f16" else "A,B ~ U[-1,1]"),
+                   "tile_config": r["cfg"]["name"]},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[head], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS[head], 4), "traffic": None,
+                     "algorithmic_bytes": alg_bytes, "flops_per_launch": flops,
+                     "kernel_ms": round(r["ev_ms"], 4)},
+        "max_rel_err": float(f"{r['rel']:.3e}"), "rel_err_limit": float(f"{r['limit']:.3e}"),
+        "parity_ok": bool(r["rel"] <= r["limit"]),
+    }
+    if "cpu" in r:
+        out["cpu_baseline"] = r["cpu"]
+    if head == "f16" and "f32" in res:
+        q = res["f32"]
+        out["also"] = {"fp32_tflops": round(flops / q["wall_ms"] * 1e-9, 2), "fp32_ms_per_step": round(q["wall_ms"], 4),
+                       "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
+                       "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
+                       "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}
+    print(json.dumps(out))
+    if not out["parity_ok"]:
+        sys.exit(3)
+
+
+if __name__ == "__main__":
+    main()

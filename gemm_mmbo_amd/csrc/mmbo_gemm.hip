@@ -90,11 +90,14 @@ double tile_cost(int dtype, int tile)
     return dtype == MMBO_F32 ? c32[tile] : c16[tile];
 }
 
-// Modelled time (arbitrary units) of running the problem with (tile, split).
+// Modelled time, in GPU clocks, of running the problem with (tile, split).
 double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, int batch)
 {
     const TileRow &r = tile_row(dtype, tile);
     const double cus = 256.0;
+    const double mac_per_clk_cu = dtype == MMBO_F32 ? 128.0 : 2048.0;   // dense MFMA rate of one CU
+    const double hbm_bytes_per_clk = 3300.0;                            // ~8 TB/s at ~2.4 GHz
+    const double esz = dtype == MMBO_F32 ? 4.0 : 2.0;
     double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch * split;
     // work-groups resident per CU, bounded by LDS (160 KB) and by 2048 threads
     int lds = dtype == MMBO_F32 ? lds_bytes_of<0, 0>(tile) : lds_bytes_of<1, 0>(tile);
@@ -108,9 +111,12 @@ double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, 
     // tiles sharing a CU share its MFMA pipes
     double conc = tiles < slots ? (tiles > cus ? tiles / cus : 1.0) : per_cu;
     double ksteps = (double)ceil_div(ceil_div(k, (size_t)split), (size_t)r.bk) * r.bk;
-    double per_tile = (double)r.bm * r.bn * (ksteps + 4.0 * r.bk) * tile_cost(dtype, tile) * conc;
-    double t = rounds * per_tile;
-    if (split > 1) t += (double)m * n * batch * (split + 2) * 64.0 / cus;   // partial-sum write + reduce pass
+    double per_tile = (double)r.bm * r.bn * (ksteps + 2.0 * r.bk) * tile_cost(dtype, tile) * conc / mac_per_clk_cu;
+    double compute = rounds * (per_tile + 1500.0);                       // + prologue/epilogue latency
+    double bytes = ((double)m * k + (double)k * n + (double)m * n) * batch * esz;
+    double t = compute > bytes / hbm_bytes_per_clk ? compute : bytes / hbm_bytes_per_clk;
+    if (split > 1)   // second launch + partial sums written and read back
+        t += 12000.0 + (double)m * n * batch * (2.0 * split * 4.0 + esz) / hbm_bytes_per_clk;
     return t;
 }
 

@@ -1,0 +1,159 @@
+"""Host-side tests of the C-ABI library: it loads, exports every symbol include/mmbo_gemm.h declares,
+validates arguments with status codes (never exit()), and its pure-host logic -- the tile-config table,
+the per-shape selection and the work-group remap -- behaves.  No compute call is made: no GPU needed.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import gemm_mmbo_amd as G
+from gemm_mmbo_amd import api
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mmbo_gemm.h")
+
+
+def test_library_is_built_in_tree_and_loads():
+    assert os.path.exists(api.LIB_PATH), "build with `python -m gemm_mmbo_amd.build`"
+    assert "gfx950" in G.version()
+
+
+def test_every_declared_symbol_is_exported():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(mmbo_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(api.EXPORTS), declared ^ set(api.EXPORTS)
+    L = ctypes.CDLL(api.LIB_PATH)
+    for name in declared:
+        assert hasattr(L, name), f"{name} declared in the header but not exported"
+
+
+def test_config_table_rows_are_consistent():
+    for dtype in (G.F32, G.F16):
+        n = G.num_configs(dtype)
+        assert n >= 6
+        names = set()
+        for cid in range(n):
+            d = G.config_info(dtype, cid)
+            names.add(d["name"])
+            assert d["threads"] % 64 == 0 and 64 <= d["threads"] <= 1024
+            assert d["macro_tile_m"] % d["wave_tile_m"] == 0 and d["macro_tile_n"] % d["wave_tile_n"] == 0
+            waves = (d["macro_tile_m"] // d["wave_tile_m"]) * (d["macro_tile_n"] // d["wave_tile_n"])
+            assert waves * 64 == d["threads"]
+            assert d["wave_tile_m"] % 32 == 0 and d["wave_tile_n"] % 32 == 0      # 32x32 MFMA blocks
+            assert 0 < d["lds_bytes"] <= 160 * 1024                                # gfx950: 160 KB per CU
+            assert d["split_k"] in (1, 2, 4, 8, 16)
+        assert len(names) == n
+    with pytest.raises(G.MmboError):
+        G.config_info(G.F32, G.num_configs(G.F32))
+    with pytest.raises(G.MmboError):
+        G.config_info(7, 0)
+
+
+def test_select_config_headline_and_skinny_shapes():
+    big16 = G.config_info(G.F16, G.select_config(G.F16, 0, 0, 8192, 8192, 8192))
+    assert big16["macro_tile_m"] * big16["macro_tile_n"] >= 256 * 128 and big16["split_k"] == 1
+    big32 = G.config_info(G.F32, G.select_config(G.F32, 0, 0, 8192, 8192, 8192))
+    assert big32["macro_tile_m"] * big32["macro_tile_n"] >= 128 * 128 and big32["split_k"] == 1
+    # 4096 x 128 x 4096 has only a few dozen large output tiles: the pick must spread the work over the
+    # 256 CUs, by smaller tiles or by splitting K
+    for dtype in (G.F32, G.F16):
+        for (m, n, k) in ((4096, 128, 4096), (128, 4096, 8192)):
+            d = G.config_info(dtype, G.select_config(dtype, 0, 0, m, n, k))
+            tiles = -(-m // d["macro_tile_m"]) * -(-n // d["macro_tile_n"]) * d["split_k"]
+            assert tiles >= 128, d
+    # tiny problem: a small tile, no split
+    d = G.config_info(G.F32, G.select_config(G.F32, 0, 0, 40, 40, 64))
+    assert d["macro_tile_m"] <= 64 and d["split_k"] == 1
+    assert G.select_config(G.F32, 0, 0, 0, 5, 5) == 0
+    with pytest.raises(G.MmboError):
+        G.select_config(3, 0, 0, 1, 1, 1)
+    with pytest.raises(G.MmboError):
+        G.select_config(G.F32, 2, 0, 1, 1, 1)
+
+
+def test_wg_remap_host_twin_matches_reference_golden():
+    """With one XCD and id = wg0 + wg1*nwg0 the kernels' mapping is the reference's WGM remap: all 29,440
+    pairs of src/gemm/ref/res."""
+    gold = np.load(os.path.join(ROOT, "tests", "golden", "wg_remap_460x64_wgm8.npy")).astype(np.int64)
+    for wg0, wg1, e0, e1 in gold:
+        assert G.wg_remap(int(wg0 + wg1 * 460), 460, 64, 8, 1) == (int(e0), int(e1))
+
+
+@pytest.mark.parametrize("nwg0,nwg1", [(32, 32), (7, 13), (1, 1), (5, 3), (16, 9), (33, 2), (2, 33)])
+@pytest.mark.parametrize("wgm,nxcd", [(8, 8), (8, 1), (4, 8), (1, 8)])
+def test_wg_remap_host_twin_bijection_and_oracle(nwg0, nwg1, wgm, nxcd):
+    seen = set()
+    for lid in range(nwg0 * nwg1):
+        t = G.wg_remap(lid, nwg0, nwg1, wgm, nxcd)
+        assert 0 <= t[0] < nwg0 and 0 <= t[1] < nwg1
+        seen.add(t)
+        if nxcd == 1:
+            assert t == O.wg_remap(lid % nwg0, lid // nwg0, nwg0, nwg1, wgm)
+    assert len(seen) == nwg0 * nwg1
+
+
+def test_wg_remap_groups_each_xcd_on_neighbouring_tiles():
+    """8192^3 with 256x256 tiles: 32 x 32 tiles.  Ids congruent mod 8 run on one XCD; the first 32 of them
+    (one per CU of that XCD) must cover a compact block: at most 8 tile columns x 4 tile rows."""
+    for x in range(8):
+        tiles = [G.wg_remap(x + 8 * i, 32, 32, 8, 8) for i in range(32)]
+        rows = {t[0] for t in tiles}
+        cols = {t[1] for t in tiles}
+        assert len(cols) <= 8 and len(rows) <= 5
+
+
+def test_wg_remap_rejects_bad_arguments():
+    with pytest.raises(G.MmboError):
+        G.wg_remap(10, 2, 5, 8, 8)          # id out of range
+    with pytest.raises(G.MmboError):
+        G.wg_remap(0, 0, 5, 8, 8)
+
+
+def _call(dtype=0, ta=0, tb=0, m=4, n=4, k=4, lda=4, ldb=4, ldc=4, A=16, B=16, C=16, cfg=-1, alpha=True, beta=True):
+    """Raw C-ABI call with fake non-null device addresses; every case here must fail validation before any
+    device work."""
+    al, be = ctypes.c_float(1.0), ctypes.c_float(0.0)
+    return api.lib().mmbo_gemm(dtype, ta, tb, m, n, k, ctypes.byref(al) if alpha else None, A, lda, B, ldb,
+                               ctypes.byref(be) if beta else None, C, ldc, cfg, None)
+
+
+def test_argument_validation_returns_status_codes():
+    assert _call(dtype=5) == 1
+    assert _call(ta=2) == 2
+    assert _call(tb=-1) == 2
+    assert _call(lda=3) == 3
+    assert _call(ta=1, k=8, lda=4) == 3          # A^T is stored k x m: lda >= k
+    assert _call(ldb=3) == 3
+    assert _call(tb=1, n=8, ldb=4, ldc=4) == 3   # B^T is stored n x k: ldb >= n
+    assert _call(ldc=3) == 3
+    assert _call(m=2 ** 31) == 3
+    assert _call(alpha=False) == 4
+    assert _call(beta=False) == 4
+    assert _call(C=None) == 4
+    assert _call(A=None) == 4
+    assert _call(cfg=10 ** 6) == 5
+    assert _call(cfg=-2) == 5
+    # empty problems succeed without touching anything (null pointers allowed)
+    assert _call(m=0, A=None, B=None, C=None, lda=1, ldc=1) == 0
+    assert _call(n=0, A=None, B=None, C=None) == 0
+    for s in range(0, 9):
+        assert api.lib().mmbo_status_string(s)
+    # strided-batched: negative batch or stride
+    al, be = ctypes.c_float(1.0), ctypes.c_float(0.0)
+    f = api.lib().mmbo_gemm_strided_batched
+    assert f(0, 0, 0, 4, 4, 4, ctypes.byref(al), 16, 4, 16, 16, 4, 16, ctypes.byref(be), 16, 4, 16, -1, -1, None) == 3
+    assert f(0, 0, 0, 4, 4, 4, ctypes.byref(al), 16, 4, -16, 16, 4, 16, ctypes.byref(be), 16, 4, 16, 2, -1, None) == 3
+    assert f(0, 0, 0, 4, 4, 4, ctypes.byref(al), 16, 4, 16, 16, 4, 16, ctypes.byref(be), 16, 4, 16, 0, -1, None) == 0
+
+
+def test_python_front_ends_keep_reference_argument_order():
+    """src/gemm/gemm.h:4-5: (m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId)."""
+    import inspect
+    want = ["m", "n", "k", "alpha", "A", "lda", "B", "ldb", "beta", "C", "ldc", "kernelId"]
+    for f in (G.naive_sgemm, G.naive_hgemm, G.sgemm_NT, G.sgemm_TN, G.hgemm_NN, G.hgemm_TT):
+        assert list(inspect.signature(f).parameters) == want

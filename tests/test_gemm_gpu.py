@@ -1,0 +1,232 @@
+"""Parity of the HIP kernels with the fp64 oracle, through the C ABI, on a real MI355X.
+
+Covers the five benchmark configurations at their full sizes, every tile config and split-K factor on
+ragged shapes, all four transposes, leading dimensions larger than the matrix, unaligned operands, the
+beta == 0 "never read C" rule, k = 0, strided batches, and size-independent properties (identity, all
+ones, linearity in alpha/beta) at full size.  Tolerances are in tests/util.py:
+fp32 <= 1e-5*sqrt(K), fp16 <= 2e-2, relative to max(|exact|, rms(exact)).
+"""
+import numpy as np
+import pytest
+
+import util as U
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32, F16 = 0, 1
+NAMES = {F32: "f32", F16: "f16"}
+
+
+def _run_and_check(p, config_id=-1, label="", offsets=(0, 0, 0)):
+    got, guard = U.run_gpu(p, config_id, offsets)
+    U.check(p, got, label)
+    assert np.all(guard == 0), "wrote past the end of C"
+    return got
+
+
+# ------------------------------------------------------------------ the five benchmark configurations
+
+def test_cfg1_sgemm_nn_1024():
+    """SGEMM NN 1024^3, ld = 1024, U[-1,1] from seed 0 (A then B from one stream), alpha=1, beta=0."""
+    p = U.Problem(F32, 0, 0, 1024, 1024, 1024, 1.0, 0.0, seed=0, c_fill="nan")
+    _run_and_check(p, label="cfg1")
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 1), (1, 0)])
+def test_cfg2_sgemm_nt_tn_4096(ta, tb):
+    """SGEMM NT and TN 4096^3, C pre-filled, alpha=1.5, beta=0.5: transposed load paths and C read-modify-write."""
+    p = U.Problem(F32, ta, tb, 4096, 4096, 4096, 1.5, 0.5, seed=2)
+    _run_and_check(p, label=f"cfg2 {'NT'[ta]}{'NT'[tb]}")
+
+
+def test_cfg3_hgemm_nn_8192():
+    """HGEMM NN 8192^3, A/B ~ N(0,1)*0.1 rounded to fp16, fp32 accumulate, alpha=1, beta=0; full check of
+    all 67M outputs against the fp64 oracle."""
+    p = U.Problem(F16, 0, 0, 8192, 8192, 8192, 1.0, 0.0, seed=3, dist="normal", c_fill="nan")
+    _run_and_check(p, label="cfg3")
+
+
+def test_cfg3_fp32_sgemm_nn_8192():
+    """The metric's fp32 leg: SGEMM NN 8192^3, U[-1,1]."""
+    p = U.Problem(F32, 0, 0, 8192, 8192, 8192, 1.0, 0.0, seed=33, c_fill="nan")
+    _run_and_check(p, label="cfg3' f32")
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+@pytest.mark.parametrize("m,n,k", [(1023, 777, 513), (4096, 128, 4096), (128, 4096, 8192)])
+def test_cfg4_irregular_and_skinny(dtype, m, n, k):
+    p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=4, c_fill="nan")
+    _run_and_check(p, label=f"cfg4 {m}x{n}x{k}")
+
+
+def test_cfg5_strided_batched_hgemm_tn():
+    """64 x (512^3) HGEMM TN, stride = one full matrix per operand, alpha=1, beta=1, C ~ U[-1,1]."""
+    p = U.Problem(F16, 1, 0, 512, 512, 512, 1.0, 1.0, batch=64, seed=5, dist="normal")
+    assert (p.sa, p.sb, p.sc) == (262144, 262144, 262144)
+    _run_and_check(p, label="cfg5")
+
+
+# ------------------------------------------------------------------ every config id on ragged shapes
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_every_config_every_transpose_ragged(dtype, ta, tb):
+    import gemm_mmbo_amd as G
+    for cid in range(G.num_configs(dtype)):
+        p = U.Problem(dtype, ta, tb, 257, 131, 1000, 1.5, 0.5, lda=None, ldc=260, seed=10 + cid)
+        _run_and_check(p, cid, label=f"config {cid} {G.config_info(dtype, cid)['name']}")
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_every_config_aligned_interior(dtype):
+    """Sizes that are multiples of every tile: only the unpredicated fast path runs."""
+    import gemm_mmbo_amd as G
+    for cid in range(G.num_configs(dtype)):
+        p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
+        _run_and_check(p, cid, label=f"config {cid}")
+
+
+# ------------------------------------------------------------------ edges
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 300, 7), (300, 1, 5), (31, 33, 2), (64, 64, 3), (5, 5, 1025),
+                                   (129, 65, 64), (33, 257, 100)])
+def test_small_and_degenerate_shapes(dtype, m, n, k):
+    for ta in (0, 1):
+        for tb in (0, 1):
+            p = U.Problem(dtype, ta, tb, m, n, k, -1.0, 1.0, seed=m * 7 + n)   # the reference's alpha=-1, beta=1
+            _run_and_check(p, label=f"{m}x{n}x{k} {'NT'[ta]}{'NT'[tb]}")
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_k_zero_scales_c_only(dtype):
+    p = U.Problem(dtype, 0, 0, 70, 50, 0, 1.0, 0.5, seed=1)
+    got = _run_and_check(p, label="k=0 beta=.5")
+    p0 = U.Problem(dtype, 0, 0, 70, 50, 0, 1.0, 0.0, seed=1, c_fill="nan")
+    got, _ = U.run_gpu(p0)
+    assert np.all(got == 0)          # alpha * (empty sum), old NaN contents not read
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_leading_dimensions_larger_than_matrix(dtype):
+    """run.sh's precedent: ldc = 44160 > M.  Padding rows of C must stay bit-identical."""
+    for (ta, tb) in ((0, 0), (0, 1), (1, 0), (1, 1)):
+        p = U.Problem(dtype, ta, tb, 384, 200, 384, -1.0, 1.0, lda=1000, ldb=777, ldc=44160 // 40, seed=6)
+        _run_and_check(p, label="ld>dim")
+        p = U.Problem(dtype, ta, tb, 100, 90, 80, 1.0, 0.0, lda=101, ldb=93, ldc=107, seed=7, c_fill="nan")
+        _run_and_check(p, label="odd ld")
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_unaligned_pointers(dtype):
+    """Device pointers offset by one element: no 128-bit access may be assumed aligned."""
+    for offs in ((1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 3, 5)):
+        p = U.Problem(dtype, 0, 0, 200, 136, 264, 1.5, 0.5, seed=8)
+        _run_and_check(p, label=f"offsets {offs}", offsets=offs)
+        p = U.Problem(dtype, 1, 1, 256, 128, 256, 1.0, 0.0, seed=9, c_fill="nan")
+        _run_and_check(p, label=f"offsets {offs} TT", offsets=offs)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_beta_zero_ignores_nan_and_inf_in_c(dtype):
+    p = U.Problem(dtype, 0, 0, 300, 200, 128, 1.0, 0.0, seed=12, c_fill="nan")
+    got, _ = U.run_gpu(p)
+    assert np.all(np.isfinite(got.astype(np.float32)))
+    p.C[:] = np.inf
+    got, _ = U.run_gpu(p, 2 + 6 * 2)          # a split-K config: the reduction must not read C either
+    assert np.all(np.isfinite(got.astype(np.float32)))
+    U.check(p, got, "beta=0 inf")
+
+
+def test_strided_batched_with_gaps_and_every_transpose():
+    for dtype in (F32, F16):
+        for (ta, tb) in ((0, 0), (0, 1), (1, 0), (1, 1)):
+            m, n, k, batch = 96, 72, 150, 5
+            p = U.Problem(dtype, ta, tb, m, n, k, 0.5, -1.0, batch=batch, seed=13,
+                          strides=(m * k + 24, k * n + 8, m * n + 40))
+            got = _run_and_check(p, label="batched gaps")
+            # the 40-element gap between C matrices is untouched
+            for b in range(batch):
+                assert np.array_equal(got[b * p.sc + m * n:(b + 1) * p.sc].view(np.uint8),
+                                      p.C[b * p.sc + m * n:(b + 1) * p.sc].view(np.uint8))
+
+
+def test_batched_equals_looped_single_calls_bitwise():
+    """Reference semantics (src/gemm/ref/Kernels.cpp:76-78,254): batch b is the same GEMM on offset pointers."""
+    import torch
+    import gemm_mmbo_amd as G
+    m, n, k, batch = 256, 192, 320, 4
+    p = U.Problem(F16, 1, 0, m, n, k, 1.0, 1.0, batch=batch, seed=14, dist="normal")
+    cid = G.select_config(F16, 1, 0, m, n, k, batch)
+    got, _ = U.run_gpu(p, cid)
+    dA, dB = torch.from_numpy(p.A).cuda(), torch.from_numpy(p.B).cuda()
+    dC = torch.from_numpy(p.C).cuda()
+    for b in range(batch):
+        G.gemm(F16, 1, 0, m, n, k, 1.0, dA.data_ptr() + 2 * b * p.sa, p.lda, dB.data_ptr() + 2 * b * p.sb, p.ldb,
+               1.0, dC.data_ptr() + 2 * b * p.sc, p.ldc, cid)
+    torch.cuda.synchronize()
+    assert np.array_equal(dC.cpu().numpy().view(np.uint16), got.view(np.uint16))
+
+
+# ------------------------------------------------------------------ size-independent properties at full size
+
+@pytest.mark.parametrize("dtype,size", [(F32, 4096), (F16, 8192)], ids=["f32-4096", "f16-8192"])
+def test_identity_and_ones_closed_forms_full_size(dtype, size):
+    """op(A) = I gives C = alpha*B exactly; all-ones operands give alpha*K exactly (K is a power of two,
+    so every partial sum is representable): bitwise checks that need no oracle run."""
+    import torch
+    import gemm_mmbo_amd as G
+    tdt = torch.float32 if dtype == F32 else torch.float16
+    n = size
+    eye = torch.eye(n, dtype=tdt, device="cuda")
+    B = torch.from_numpy(O.fill_uniform(n * n, dtype, 21)).cuda()
+    C = torch.full((n * n,), float("nan"), dtype=tdt, device="cuda")
+    for (ta, tb) in ((0, 0), (1, 0)):
+        G.gemm(dtype, ta, tb, n, n, n, 1.0, eye, n, B, n, 0.0, C, n)
+        torch.cuda.synchronize()
+        assert torch.equal(C, B)
+    ones = torch.ones(n * n, dtype=tdt, device="cuda")
+    G.gemm(dtype, 0, 1, n, n, n, 0.25, ones, n, ones, n, 0.0, C, n)
+    torch.cuda.synchronize()
+    assert torch.all(C == 0.25 * n)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_linearity_in_alpha_and_beta(dtype):
+    """gemm(2a, 2b) == 2 * gemm(a, b) bit for bit: scaling by two is exact in binary floating point
+    (outside the fp16 subnormal range, where the doubled value has one more significant bit to round)."""
+    p = U.Problem(dtype, 0, 1, 1000, 600, 700, 0.75, -0.5, seed=30, dist="normal")
+    g1, _ = U.run_gpu(p)
+    p2 = U.Problem(dtype, 0, 1, 1000, 600, 700, 1.5, -1.0, seed=30, dist="normal")
+    g2, _ = U.run_gpu(p2)
+    doubled = (g1.astype(np.float32) * 2).astype(g1.dtype)
+    normal = np.abs(g2.astype(np.float32)) >= 2.0 ** -13
+    assert normal.mean() > 0.99
+    assert np.array_equal(doubled[normal], g2[normal])
+
+
+def test_repeatable_bitwise_including_split_k():
+    """Split-K partials are reduced in a fixed order: two runs give identical bits."""
+    import gemm_mmbo_amd as G
+    for dtype in (F32, F16):
+        p = U.Problem(dtype, 0, 0, 4096, 128, 4096, 1.0, 0.0, seed=31, c_fill="nan")
+        for cid in (G.select_config(dtype, 0, 0, 4096, 128, 4096), 2 + 6 * 3):
+            a, _ = U.run_gpu(p, cid)
+            b, _ = U.run_gpu(p, cid)
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def test_async_on_user_stream():
+    """The launch goes to the caller's stream (reference: null stream only, src/gemm/common.h:12)."""
+    import torch
+    import gemm_mmbo_amd as G
+    p = U.Problem(F32, 0, 0, 512, 512, 512, 1.0, 0.0, seed=32, c_fill="nan")
+    s = torch.cuda.Stream()
+    dA, dB, dC = (torch.from_numpy(x).cuda() for x in (p.A, p.B, p.C))
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        G.gemm(F32, 0, 0, 512, 512, 512, 1.0, dA, 512, dB, 512, 0.0, dC, 512, -1, s)
+    s.synchronize()
+    U.check(p, dC.cpu().numpy(), "stream")

@@ -73,7 +73,7 @@ def run_gpu(p, config_id=-1, offset_elems=(0, 0, 0)):
     import gemm_mmbo_amd as G
 
     def up(h, off):
-        t = torch.empty(h.size + off + 8, dtype=torch.float32 if p.dtype == F32 else torch.float16, device="cuda")
+        t = torch.zeros(h.size + off + 8, dtype=torch.float32 if p.dtype == F32 else torch.float16, device="cuda")
         t[off:off + h.size].copy_(torch.from_numpy(h))
         return t
 
