@@ -14,7 +14,20 @@
 
 namespace mmbo {
 
+hipError_t launch_hgemm_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream);
+
 namespace {
+
+// Config ids: [0, NUM_TILES*NUM_SPLITS) are the staged kernel's (tile, split) pairs; fp16 has one more,
+// the direct-to-LDS ring kernel, usable when m, n are multiples of 256, k of 32 and operands aligned.
+constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
+constexpr int kRingConfig = kStagedConfigs;
+inline int num_configs_of(int dtype) { return dtype == MMBO_F16 ? kStagedConfigs + 1 : kStagedConfigs; }
+
+inline bool ring_eligible(int dtype, size_t m, size_t n, size_t k)
+{
+    return dtype == MMBO_F16 && m % 256 == 0 && n % 256 == 0 && k % 32 == 0 && k >= 32;
+}
 
 thread_local int g_last_hip_error = 0;
 
@@ -160,17 +173,23 @@ const char *mmbo_status_string(int status)
 int mmbo_num_configs(int dtype)
 {
     if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
-    return NUM_TILES * NUM_SPLITS;
+    return num_configs_of(dtype);
 }
 
 int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
 {
     if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
     if (!out) return MMBO_ERR_NULL_POINTER;
-    if (config_id < 0 || config_id >= NUM_TILES * NUM_SPLITS) return MMBO_ERR_INVALID_CONFIG;
+    if (config_id < 0 || config_id >= num_configs_of(dtype)) return MMBO_ERR_INVALID_CONFIG;
+    std::memset(out, 0, sizeof(*out));
+    if (config_id == kRingConfig) {
+        std::snprintf(out->name, sizeof(out->name), "MT256x256x32_WT064x128_W8_GSU01_DTL1_RING5");
+        out->macro_tile_m = 256; out->macro_tile_n = 256; out->depth_u = 32; out->threads = 512;
+        out->wave_tile_m = 64; out->wave_tile_n = 128; out->split_k = 1; out->lds_bytes = 160 * 1024;
+        return MMBO_OK;
+    }
     int tile = config_id % NUM_TILES, split = kSplits[config_id / NUM_TILES];
     const TileRow &r = tile_row(dtype, tile);
-    std::memset(out, 0, sizeof(*out));
     std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d", r.bm, r.bn, r.bk,
                   r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, split);
     out->macro_tile_m = r.bm;
@@ -201,6 +220,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
             if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
         }
     }
+    // the ring kernel replaces the big staged tiles wherever it applies
+    if (ring_eligible(dtype, m, n, k) && best < NUM_TILES && best <= 1) best = kRingConfig;
     return best;
 }
 
@@ -254,7 +275,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
             return MMBO_ERR_INVALID_SIZE;
     }
     if (strideA < 0 || strideB < 0 || strideC < 0) return MMBO_ERR_INVALID_SIZE;
-    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= NUM_TILES * NUM_SPLITS))
+    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= num_configs_of(dtype)))
         return MMBO_ERR_INVALID_CONFIG;
     if (m == 0 || n == 0 || batch == 0) return MMBO_OK;          // nothing to write
     if (!C) return MMBO_ERR_NULL_POINTER;
@@ -267,6 +288,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
     }
+    const bool use_ring = config_id == kRingConfig;
+    if (use_ring) config_id = 0;                                // same macro tile as staged row 0, no split
     int tile = config_id % NUM_TILES;
     int split = kSplits[config_id / NUM_TILES];
     const TileRow &r = tile_row(dtype, tile);
@@ -310,6 +333,11 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     a.vec_c = aligned16(C, ldc, strideC);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (use_ring) {
+        if (!ring_eligible(dtype, m, n, k) || !a.vec_a || !a.vec_b) return MMBO_ERR_INVALID_CONFIG;
+        hipError_t e = launch_hgemm_ring(transA, transB, a, s);
+        return e == hipSuccess ? MMBO_OK : hip_fail(e);
+    }
     if (split > 1) {
         size_t bytes = (size_t)split * batch * m * n * sizeof(float);
         int rc = workspace(bytes, &a.ws);

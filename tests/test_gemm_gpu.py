@@ -76,6 +76,12 @@ def test_every_config_every_transpose_ragged(dtype, ta, tb):
     import gemm_mmbo_amd as G
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, ta, tb, 257, 131, 1000, 1.5, 0.5, lda=None, ldc=260, seed=10 + cid)
+        if "DTL1" in G.config_info(dtype, cid)["name"]:
+            # the direct-to-LDS kernel only takes whole 256 x 256 x 32 tiles: a ragged shape must be refused
+            with pytest.raises(G.MmboError) as e:
+                U.run_gpu(p, cid)
+            assert e.value.status == 5
+            continue
         _run_and_check(p, cid, label=f"config {cid} {G.config_info(dtype, cid)['name']}")
 
 
@@ -86,6 +92,25 @@ def test_every_config_aligned_interior(dtype):
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
         _run_and_check(p, cid, label=f"config {cid}")
+
+
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_direct_to_lds_ring_kernel_every_transpose(ta, tb):
+    """The HGEMM fast path (global->LDS direct loads through a five-deep ring) by explicit config id: short and
+    long K (fewer slices than ring buffers, odd slice counts), beta read-modify-write, ld > dim, batches."""
+    import gemm_mmbo_amd as G
+    cid = G.num_configs(F16) - 1
+    assert "DTL1" in G.config_info(F16, cid)["name"]
+    for (m, n, k, alpha, beta, batch) in ((256, 256, 32, 1.0, 0.0, 1), (512, 256, 96, 1.5, 0.5, 1), (256, 768, 160, 1.0, 0.0, 1),
+                                          (768, 1024, 1056, -1.0, 1.0, 1), (256, 512, 4096, 1.0, 0.0, 1), (256, 256, 224, 1.0, 1.0, 3)):
+        p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=70 + k, dist="normal",
+                      c_fill="uniform" if beta else "nan")
+        _run_and_check(p, cid, label=f"ring {m}x{n}x{k} b{batch}")
+    p = U.Problem(F16, ta, tb, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71, dist="normal")
+    _run_and_check(p, cid, label="ring ld>dim")
+    # the per-shape table picks it for the headline shape
+    assert G.select_config(F16, ta, tb, 8192, 8192, 8192) == cid
 
 
 # ------------------------------------------------------------------ edges
@@ -230,3 +255,36 @@ def test_async_on_user_stream():
         G.gemm(F32, 0, 0, 512, 512, 512, 1.0, dA, 512, dB, 512, 0.0, dC, 512, -1, s)
     s.synchronize()
     U.check(p, dC.cpu().numpy(), "stream")
+
+
+# ------------------------------------------------------------------ C++ harness shaped like the reference's
+
+def _harness(path, *args):
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, path)
+    if not os.path.exists(exe):
+        pytest.skip(f"{path} not built (run __graft_entry__.build())")
+    return subprocess.run([exe, *map(str, args)], capture_output=True, text=True, timeout=280)
+
+
+def test_cpp_verify_main_reference_defaults_and_failure_exit_code():
+    """tests/harness/test: the reference's test.cc flow (NT, alpha=-1, beta=1, M=44160 N=2048 K=384) through the
+    C++ front-ends; exit status 0 only when every element matches the oracle."""
+    r = _harness("tests/harness/test")
+    assert r.returncode == 0 and "result check passed" in r.stdout, r.stdout + r.stderr
+    r = _harness("tests/harness/test", 1023, 777, 513, "N", "N", "h", 1, 0)
+    assert r.returncode == 0 and "result check passed" in r.stdout, r.stdout + r.stderr
+    r = _harness("tests/harness/test", 64, 64, 64, "N", "N", "s", 1, 0, 999)      # bad kernelId: error, not exit(0)
+    assert r.returncode != 0
+
+
+def test_cpp_benchmark_main_modes():
+    """gemm_mmbo_amd/host/benchmark: `type M N K lda ldb ldc` like the reference's; type 1 sweeps every config."""
+    r = _harness("gemm_mmbo_amd/host/benchmark", 0, 1024, 1024, 1024, 1024, 1024, 1024, "N", "N", "s", 1, 1, 0)
+    assert r.returncode == 0 and "sgemm(NN): kernel" in r.stdout, r.stdout + r.stderr
+    r = _harness("gemm_mmbo_amd/host/benchmark", 1, 512, 512, 512, 512, 512, 512, "T", "N", "h", 4, 1, 1)
+    assert r.returncode == 0 and "hgemm(TN): kernel" in r.stdout, r.stdout + r.stderr
+    r = _harness("gemm_mmbo_amd/host/benchmark", 0, 64, 64)
+    assert r.returncode == 2
