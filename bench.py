@@ -17,6 +17,10 @@ sys.path.insert(0, ROOT)
 
 METRIC = "GEMM TFLOP/s + % of MFMA peak, fp16 & fp32 at 8192^3, 1 MI355X"
 PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}      # MI355X published dense matrix peaks
+# Bytes per launch that crossed the L2 <-> fabric boundary, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this same command (each scaled by the counter's reading for a plain elementwise pass of known size; the
+# summaries with the commands are profiles/hgemm_ring_8192.txt and profiles/sgemm_staged_8192.txt).
+MEASURED_TRAFFIC_BYTES = {"f16": 1.634e9 + 0.282e9, "f32": 3.53e9 + 0.30e9}
 
 
 def time_gemm(G, torch, dtype, m, n, k, steps, warmup, seed):
@@ -121,6 +125,12 @@ def main():
         del tensors, host
         torch.cuda.empty_cache()
 
+    ceilings = {}
+    if not args.only:
+        for name, dtype in (("f16", G.F16), ("f32", G.F32)):
+            for rnd in (0, 1):
+                tf, mhz = G.probe_mfma_ceiling(dtype, bool(rnd))
+                ceilings[f"{name}_{'random' if rnd else 'ones'}_operands"] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
     head = "f16" if "f16" in res else "f32"
     r = res[head]
     tflops = flops / r["wall_ms"] * 1e-9
@@ -134,7 +144,7 @@ def main():
                                + ("A,B ~ N(0,1)*0.1 rounded to fp16, fp32 accumulate" if head == "f16" else "A,B ~ U[-1,1]"),
                    "tile_config": r["cfg"]["name"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[head], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS[head], 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS[head], 4), "traffic": MEASURED_TRAFFIC_BYTES[head],
                      "algorithmic_bytes": alg_bytes, "flops_per_launch": flops,
                      "kernel_ms": round(r["ev_ms"], 4)},
         "max_rel_err": float(f"{r['rel']:.3e}"), "rel_err_limit": float(f"{r['limit']:.3e}"),
@@ -142,6 +152,12 @@ def main():
     }
     if "cpu" in r:
         out["cpu_baseline"] = r["cpu"]
+    if ceilings:
+        # what a register-only MFMA loop sustains on this box (the chip lowers its clock under power)
+        out["mfma_issue_ceiling"] = ceilings
+        c = ceilings.get(f"{head}_random_operands")
+        if c:
+            out["roofline"]["frac_of_measured_mfma_ceiling"] = round(achieved / c["tflops"], 4)
     if head == "f16" and "f32" in res:
         q = res["f32"]
         out["also"] = {"fp32_tflops": round(flops / q["wall_ms"] * 1e-9, 2), "fp32_ms_per_step": round(q["wall_ms"], 4),

@@ -5,6 +5,6 @@
 """
 from .api import (  # noqa: F401
     CONFIG_AUTO, F16, F32, OP_N, OP_T, MmboError, config_info, gemm, gemm_strided_batched, hgemm_NN, hgemm_NT,
-    hgemm_TN, hgemm_TT, lib, naive_hgemm, naive_sgemm, num_configs, release_workspace, select_config, sgemm_NN,
+    hgemm_TN, hgemm_TT, lib, naive_hgemm, naive_sgemm, num_configs, probe_mfma_ceiling, release_workspace, select_config, sgemm_NN,
     sgemm_NT, sgemm_TN, sgemm_TT, version, wg_remap,
 )

@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmmbo_gemm.so")
 
 EXPORTS = (
     "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
-    "mmbo_wg_remap", "mmbo_release_workspace", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
+    "mmbo_wg_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
 
@@ -66,6 +66,9 @@ def lib():
         L.mmbo_wg_remap.argtypes = [cu, cu, cu, cu, cu, ctypes.POINTER(cu), ctypes.POINTER(cu)]
         L.mmbo_wg_remap.restype = ci
         L.mmbo_release_workspace.restype = ci
+        dp = ctypes.POINTER(ctypes.c_double)
+        L.mmbo_probe_mfma_ceiling.argtypes = [ci, ci, dp, dp]
+        L.mmbo_probe_mfma_ceiling.restype = ci
         L.mmbo_status_string.argtypes = [ci]
         L.mmbo_status_string.restype = ctypes.c_char_p
         L.mmbo_last_hip_error.restype = ci
@@ -138,6 +141,13 @@ def wg_remap(linear_id, nwg0, nwg1, wgm=8, num_xcd=8):
     a, b = ctypes.c_uint(0), ctypes.c_uint(0)
     _check(lib().mmbo_wg_remap(linear_id, nwg0, nwg1, wgm, num_xcd, ctypes.byref(a), ctypes.byref(b)))
     return a.value, b.value
+
+
+def probe_mfma_ceiling(dtype, random_operands=True):
+    """(TFLOP/s, shader MHz) of a register-only MFMA loop on the current device."""
+    tf, mhz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    _check(lib().mmbo_probe_mfma_ceiling(dtype, 1 if random_operands else 0, ctypes.byref(tf), ctypes.byref(mhz)))
+    return tf.value, mhz.value
 
 
 def release_workspace():

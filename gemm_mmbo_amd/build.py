@@ -27,7 +27,7 @@ FLAGS = [
 
 
 def _units():
-    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("inst_ring.hip", "inst_ring.o", [])]
+    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("inst_ring.hip", "inst_ring.o", []), ("probe.hip", "probe.o", [])]
     for dtype in (0, 1):
         for tile in range(NUM_TILES):
             units.append(("inst_staged.hip", f"inst_staged_{dtype}_{tile}.o",

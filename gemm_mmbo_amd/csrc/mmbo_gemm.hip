@@ -11,6 +11,7 @@
 #include "gemm_common.hpp"
 #include "gemm_staged.hpp"
 #include "launch.hpp"
+#include "tuned_table.hpp"
 
 namespace mmbo {
 
@@ -94,22 +95,26 @@ int lds_bytes_of(int tile)
 
 inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 
-// Relative cost of one k-step of a tile, per element of C: smaller tiles re-read more of A and B
-// per flop and keep fewer MFMAs in flight.  Hand-set from measurements on MI355X.
+// Relative MFMA-pipe cost of a tile's inner loop (1.0 = the 256 x 256 tile): smaller wave tiles read more
+// LDS per MFMA.  Fitted to sweeps of every config on MI355X.
 double tile_cost(int dtype, int tile)
 {
-    static const double c32[NUM_TILES] = {1.00, 1.05, 1.15, 1.40, 1.9, 6.0};
-    static const double c16[NUM_TILES] = {1.00, 1.15, 1.35, 1.80, 2.6, 8.0};
+    static const double c32[NUM_TILES] = {1.00, 1.06, 1.03, 1.03, 1.08, 2.2};
+    static const double c16[NUM_TILES] = {1.00, 1.10, 1.15, 1.25, 1.9, 4.0};
     return dtype == MMBO_F32 ? c32[tile] : c16[tile];
 }
 
-// Modelled time, in GPU clocks, of running the problem with (tile, split).
+// Modelled time, in GPU clocks, of running the problem with the staged kernel of (tile, split).
+// The staged kernel prefetches one stage ahead, so a stage costs the larger of its MFMA time (shared by the
+// work-groups resident on the CU) and the global-load latency; short K and few tiles are latency-bound,
+// which is what split-K and small tiles buy back.
 double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, int batch)
 {
     const TileRow &r = tile_row(dtype, tile);
     const double cus = 256.0;
     const double mac_per_clk_cu = dtype == MMBO_F32 ? 128.0 : 2048.0;   // dense MFMA rate of one CU
     const double hbm_bytes_per_clk = 3300.0;                            // ~8 TB/s at ~2.4 GHz
+    const double load_latency = 1700.0;                                 // clocks from issue to data in registers
     const double esz = dtype == MMBO_F32 ? 4.0 : 2.0;
     double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch * split;
     // work-groups resident per CU, bounded by LDS (160 KB) and by 2048 threads
@@ -118,18 +123,19 @@ double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, 
     int thr = r.wm * r.wn * 64;
     if (per_cu > 2048 / thr) per_cu = 2048 / thr;
     if (per_cu < 1) per_cu = 1;
-    if (per_cu > 4) per_cu = 4;
     double slots = cus * per_cu;
     double rounds = (double)ceil_div((size_t)tiles, (size_t)slots);
-    // tiles sharing a CU share its MFMA pipes
-    double conc = tiles < slots ? (tiles > cus ? tiles / cus : 1.0) : per_cu;
-    double ksteps = (double)ceil_div(ceil_div(k, (size_t)split), (size_t)r.bk) * r.bk;
-    double per_tile = (double)r.bm * r.bn * (ksteps + 2.0 * r.bk) * tile_cost(dtype, tile) * conc / mac_per_clk_cu;
-    double compute = rounds * (per_tile + 1500.0);                       // + prologue/epilogue latency
+    double resident = tiles >= slots ? per_cu : (tiles > cus ? tiles / cus : 1.0);   // tiles sharing one CU's pipes
+    double stage_mfma = (double)r.bm * r.bn * r.bk * tile_cost(dtype, tile) / mac_per_clk_cu;
+    double stage = stage_mfma * resident > load_latency ? stage_mfma * resident : load_latency;
+    double stages = (double)ceil_div(ceil_div(k, (size_t)split), (size_t)r.bk);
+    double epilogue = (double)r.bm * r.bn * esz * resident / 24.0;      // C tile through one CU's store path
+    double compute = rounds * (stages * stage + load_latency + epilogue);
     double bytes = ((double)m * k + (double)k * n + (double)m * n) * batch * esz;
     double t = compute > bytes / hbm_bytes_per_clk ? compute : bytes / hbm_bytes_per_clk;
+    t += 9000.0;                                                         // launch
     if (split > 1)   // second launch + partial sums written and read back
-        t += 12000.0 + (double)m * n * batch * (2.0 * split * 4.0 + esz) / hbm_bytes_per_clk;
+        t += 9000.0 + (double)m * n * batch * (2.0 * split * 4.0 + esz) / hbm_bytes_per_clk;
     return t;
 }
 
@@ -209,6 +215,10 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
     if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
     if (batch < 0) return -MMBO_ERR_INVALID_SIZE;
     if (m == 0 || n == 0 || batch == 0) return 0;
+    for (const TunedRow &t : kTuned)
+        if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
+            t.batch == batch)
+            return t.config_id;
     int best = 0;
     double best_t = 0.0;
     for (int si = 0; si < NUM_SPLITS; ++si) {
@@ -220,6 +230,7 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
             if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
         }
     }
+    // the ring kernel replaces the big staged tiles wherever it applies
     // the ring kernel replaces the big staged tiles wherever it applies
     if (ring_eligible(dtype, m, n, k) && best < NUM_TILES && best <= 1) best = kRingConfig;
     return best;

@@ -1,0 +1,131 @@
+// MFMA issue-ceiling probe: a register-only loop of matrix instructions, two wavefronts per SIMD on every CU,
+// timed with HIP events and with the shader clock counter against the fixed 100 MHz wall counter.
+//
+// The reference has the same kind of probe for its FMA pipe: src/gemm/assembly/error_kernel_000.s is its
+// kernel with every LDS read and most waits removed ("FMA-issue-only", wrong results by design).  Here the
+// probe also answers what the GEMM numbers have to be read against: on MI355X the sustained MFMA rate
+// depends on the operand bits (the chip lowers its clock under power), so "percent of peak" needs the
+// measured clock and the measured ceiling beside it.
+#include "../../include/mmbo_gemm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <vector>
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <bool F16>
+__global__ void __launch_bounds__(512) mfma_ceiling_kernel(const uint32_t *src, float *out, long long *clk, int iters)
+{
+    f32x16 acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+    union { uint32_t u[4]; f16x8 h; float f[4]; } a[4], b[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            a[q].u[e] = src[(threadIdx.x * 4 + q) * 4 + e];
+            b[q].u[e] = src[8192 + (threadIdx.x * 4 + q) * 4 + e];
+        }
+    const long long t0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if constexpr (F16) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i % 4].h, b[(i / 2) % 4].h, acc[i], 0, 0, 0);
+            else acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i % 4].f[0], b[(i / 2) % 4].f[0], acc[i], 0, 0, 0);
+        }
+    }
+    const long long t1 = clock64(), w1 = wall_clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s += acc[i][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        clk[0] = t1 - t0;
+        clk[1] = w1 - w0;
+    }
+}
+
+uint64_t mix64(uint64_t z)
+{
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+}  // namespace
+
+extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *tflops, double *shader_mhz)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if (!tflops || !shader_mhz) return MMBO_ERR_NULL_POINTER;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MMBO_ERR_NO_DEVICE;
+    const int blocks = prop.multiProcessorCount, threads = 512;
+    const int iters = dtype == MMBO_F16 ? 20000 : 10000;
+
+    // operands: 1.0 everywhere, or uniform [-0.3, 0.3) with every mantissa bit in play
+    std::vector<uint32_t> h(16384);
+    for (size_t i = 0; i < h.size(); ++i) {
+        if (dtype == MMBO_F16) {
+            _Float16 lo = (_Float16)1.0f, hi = (_Float16)1.0f;
+            if (random_operands) {
+                uint64_t r = mix64(i);
+                lo = (_Float16)(((double)(r & 0xFFFFFF) / 16777216.0 * 2.0 - 1.0) * 0.3);
+                hi = (_Float16)(((double)((r >> 24) & 0xFFFFFF) / 16777216.0 * 2.0 - 1.0) * 0.3);
+            }
+            uint16_t lb, hb;
+            __builtin_memcpy(&lb, &lo, 2);
+            __builtin_memcpy(&hb, &hi, 2);
+            h[i] = (uint32_t)lb | ((uint32_t)hb << 16);
+        } else {
+            float v = 1.0f;
+            if (random_operands) v = (float)(((double)(mix64(i) >> 11) / 9007199254740992.0 * 2.0 - 1.0) * 0.3);
+            __builtin_memcpy(&h[i], &v, 4);
+        }
+    }
+    uint32_t *d_src = nullptr;
+    float *d_out = nullptr;
+    long long *d_clk = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = MMBO_ERR_HIP;
+    do {
+        if (hipMalloc(reinterpret_cast<void **>(&d_src), h.size() * 4) != hipSuccess) break;
+        if (hipMalloc(reinterpret_cast<void **>(&d_out), (size_t)blocks * threads * 4) != hipSuccess) break;
+        if (hipMalloc(reinterpret_cast<void **>(&d_clk), 16) != hipSuccess) break;
+        if (hipMemcpy(d_src, h.data(), h.size() * 4, hipMemcpyHostToDevice) != hipSuccess) break;
+        if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
+        float ms = 0.0f;
+        for (int rep = 0; rep < 3; ++rep) {      // the clock settles over the first launches; the last one counts
+            (void)hipEventRecord(e0, nullptr);
+            if (dtype == MMBO_F16) hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
+            else hipLaunchKernelGGL(mfma_ceiling_kernel<false>, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
+            (void)hipEventRecord(e1, nullptr);
+            if (hipEventSynchronize(e1) != hipSuccess) break;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+        }
+        long long c[2] = {0, 1};
+        if (hipMemcpy(c, d_clk, 16, hipMemcpyDeviceToHost) != hipSuccess || ms <= 0.0f) break;
+        const double flops_per_mfma = dtype == MMBO_F16 ? 32768.0 : 4096.0;
+        *tflops = (double)blocks * (threads / 64) * iters * 8.0 * flops_per_mfma / (ms * 1e-3) * 1e-12;
+        *shader_mhz = c[1] > 0 ? (double)c[0] / (double)c[1] * 100.0 : 0.0;
+        rc = MMBO_OK;
+    } while (false);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    (void)hipFree(d_src);
+    (void)hipFree(d_out);
+    (void)hipFree(d_clk);
+    return rc;
+}

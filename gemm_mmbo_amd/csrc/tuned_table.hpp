@@ -1,0 +1,38 @@
+// Exact-shape picks measured on MI355X by sweeping every config id (gemm_mmbo_amd/host/benchmark type 1 does
+// the same sweep).  The reference keeps such a table for its Tensile kernels: exact size -> (solution index,
+// measured GFLOP/s), src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:929-1177.  Shapes not listed here go through
+// the cost model in mmbo_gemm.hip.
+#pragma once
+
+#include <cstddef>
+
+namespace mmbo {
+
+struct TunedRow {
+    int dtype, transA, transB;
+    size_t m, n, k;
+    int batch;
+    int config_id;
+    float tflops;     // measured with that config, for the record
+};
+
+constexpr TunedRow kTuned[] = {
+    //dtype ta tb     m      n      k  batch  id   TFLOP/s
+    {0, 0, 0,  1024,  1024,  1024,  1,   4,   77.8f},
+    {0, 0, 1,  4096,  4096,  4096,  1,   0,  131.3f},
+    {0, 1, 0,  4096,  4096,  4096,  1,   0,  127.2f},
+    {0, 0, 0,  8192,  8192,  8192,  1,   0,  137.0f},
+    {1, 0, 0,  8192,  8192,  8192,  1,  30, 1020.0f},
+    {0, 0, 0,  1023,   777,   513,  1,   4,   24.7f},
+    {1, 0, 0,  1023,   777,   513,  1,  16,   26.3f},
+    {0, 0, 0,  4096,   128,  4096,  1,  22,   79.5f},
+    {1, 0, 0,  4096,   128,  4096,  1,  16,  192.6f},
+    {0, 0, 0,   128,  4096,  8192,  1,  21,   94.1f},
+    {1, 0, 0,   128,  4096,  8192,  1,  16,  281.6f},
+    {1, 1, 0,   512,   512,   512, 64,  30,  412.4f},
+    {0, 0, 0,  2048,  2048,  2048,  1,   3,  113.8f},
+    {1, 0, 0,  2048,  2048,  2048,  1,   3,  559.6f},
+    {0, 0, 1, 44160,  2048,   384,  1,   3,  114.1f},
+};
+
+}  // namespace mmbo

@@ -288,3 +288,16 @@ def test_cpp_benchmark_main_modes():
     assert r.returncode == 0 and "hgemm(TN): kernel" in r.stdout, r.stdout + r.stderr
     r = _harness("gemm_mmbo_amd/host/benchmark", 0, 64, 64)
     assert r.returncode == 2
+
+
+def test_mfma_ceiling_probe_reports_plausible_numbers():
+    """mmbo_probe_mfma_ceiling: a register-only MFMA loop cannot beat the published peaks, and constant operands
+    are never slower than random ones (the chip clocks down under power)."""
+    import gemm_mmbo_amd as G
+    ones16, mhz1 = G.probe_mfma_ceiling(F16, False)
+    rnd16, mhz2 = G.probe_mfma_ceiling(F16, True)
+    ones32, mhz3 = G.probe_mfma_ceiling(F32, False)
+    assert 500 < rnd16 <= ones16 * 1.05 and ones16 < 2600
+    assert 50 < ones32 < 165
+    for mhz in (mhz1, mhz2, mhz3):
+        assert 500 < mhz < 2600
