@@ -16,6 +16,7 @@ OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(CSRC, "libmmbo_gemm.so")
 
 NUM_TILES = 6  # keep in step with csrc/configs.hpp
+NUM_RING_TILES = 4
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -27,10 +28,13 @@ FLAGS = [
 
 
 def _units():
-    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("inst_ring.hip", "inst_ring.o", []), ("probe.hip", "probe.o", [])]
+    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("probe.hip", "probe.o", [])]
     for dtype in (0, 1):
         for tile in range(NUM_TILES):
             units.append(("inst_staged.hip", f"inst_staged_{dtype}_{tile}.o",
+                          [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
+        for tile in range(NUM_RING_TILES):
+            units.append(("inst_ring.hip", f"inst_ring_{dtype}_{tile}.o",
                           [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
     extra = os.path.join(CSRC, "extra_units.txt")
     if os.path.exists(extra):

@@ -36,4 +36,20 @@ constexpr TileRow kTilesF16[NUM_TILES] = {
 
 constexpr const TileRow &tile_row(int dtype, int tile) { return dtype == 0 ? kTilesF32[tile] : kTilesF16[tile]; }
 
+// Ring kernel tiles (gemm_ring.hpp), the same for both element types; depthU is 32 (fp16) / 16 (fp32).
+// Config ids continue after the staged ones:  NUM_TILES*NUM_SPLITS + ring_tile + NUM_RING_TILES * split_index.
+struct RingRow {
+    int bm, bn;
+    int wm, wn;       // wavefronts along M and N (swapped for TT so the transposed-read operand has fewer fragments)
+    int depth;        // LDS ring buffers
+};
+constexpr int NUM_RING_TILES = 4;
+constexpr RingRow kRingTiles[NUM_RING_TILES] = {
+    {256, 256, 4, 2, 5},     // 160 KB of LDS, one work-group per CU
+    {128, 128, 2, 2, 5},     //  80 KB, two per CU
+    {128,  64, 2, 2, 6},     //  72 KB, two per CU
+    { 64,  64, 2, 2, 6},     //  48 KB, three per CU
+};
+constexpr int ring_bk(int dtype) { return dtype == 0 ? 16 : 32; }
+
 }  // namespace mmbo

@@ -84,4 +84,86 @@ template <> struct ElemTraits<half_t> {
     static constexpr int PAD_RC = 32;  // 64 B: the four k-rows of one transposed read land in distinct bank groups
 };
 
+// Write-back of one wavefront's FM x FN blocks of 32 x 32 accumulators.
+//   acc[i][j][4*q + r] is C(row, col) with  row = wrow0 + i*32 + 8*q + 4*(lane/32) + r,  col = wcol0 + j*32 + lane%32
+// (the v_mfma_f32_32x32 result layout: a lane holds four consecutive rows of one column, four times).
+// With GlobalSplitU > 1 the raw sums go to the fp32 workspace [split][batch][n][m] and the reduction kernel
+// applies alpha and beta.  Otherwise  C = alpha*acc (+ beta*C): the old C is read only when beta != 0
+// (reference: src/gemm/ref/Kernels.cpp:87, guarded stores :1064-1121; order of operations alpha*acc first, then
+// fma(beta, C, .), as the reference's assembly epilogue does).  INTERIOR = true drops the m/n guards.
+template <typename T, int FM, int FN, bool INTERIOR>
+__device__ inline void write_back(const f32x16 (&acc)[FM][FN], const GemmArgs &args, uint32_t wrow0, uint32_t wcol0,
+                                  uint32_t batch, uint32_t split, int lane)
+{
+    constexpr int ESZ = sizeof(T);
+    const uint32_t m = args.m, n = args.n;
+    const int g = lane >> 5, cl = lane & 31;
+    if (args.splits > 1) {
+        float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)m * n;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                uint32_t col = wcol0 + j * 32 + cl;
+                if (!INTERIOR && col >= n) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t row = wrow0 + i * 32 + 8 * q + 4 * g;
+                    float *p = ws + (size_t)col * m + row;
+                    if (INTERIOR || (row + 4 <= m && (m & 3) == 0)) {
+                        *reinterpret_cast<f32x4 *>(p) =
+                            f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (row + r < m) p[r] = acc[i][j][4 * q + r];
+                    }
+                }
+            }
+        return;
+    }
+
+    const float alpha = args.alpha, beta = args.beta;
+    const uint32_t ldc = args.ldc;
+    T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
+    const bool vec_c = args.vec_c != 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            uint32_t col = wcol0 + j * 32 + cl;
+            if (!INTERIOR && col >= n) continue;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t row = wrow0 + i * 32 + 8 * q + 4 * g;
+                if (!INTERIOR && row >= m) continue;
+                T *p = C + (size_t)col * ldc + row;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * q + r];
+                if (vec_c && (INTERIOR || row + 4 <= m)) {
+                    union { T e[4]; u32x4 v4; u32x2 v2; } io;
+                    if (beta != 0.0f) {                       // beta == 0: C is never read
+                        if constexpr (ESZ == 4) io.v4 = *reinterpret_cast<const u32x4 *>(p);
+                        else io.v2 = *reinterpret_cast<const u32x2 *>(p);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) io.e[r] = (T)v[r];
+                    if constexpr (ESZ == 4) *reinterpret_cast<u32x4 *>(p) = io.v4;
+                    else *reinterpret_cast<u32x2 *>(p) = io.v2;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (INTERIOR || row + r < m) {
+                            float o = v[r];
+                            if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
+                            p[r] = (T)o;
+                        }
+                }
+            }
+        }
+}
+
 }  // namespace mmbo

@@ -1,21 +1,19 @@
-// HGEMM fast path for gfx950: 256 x 256 macro tile, 8 wavefronts, K consumed in slices of 32 through a
-// five-deep ring of LDS buffers filled by global->LDS direct loads, fragments double-buffered in registers.
+// Ring kernel for gfx950: the fast path for problems made of whole tiles (m % BM == 0, n % BN == 0,
+// k % BK == 0 per split, A and B 16-byte aligned).  Everything else takes the staged kernel.
 //
-// It serves problems whose m and n are multiples of 256, k a multiple of 32, and whose operands are
-// 16-byte aligned; everything else takes the staged kernel (gemm_staged.hpp).
+// K is consumed in slices of 64 bytes per row (BK = 32 halves / 16 floats) through a DEPTH-deep ring of LDS
+// buffers filled by global->LDS direct loads; MFMA operand fragments are double-buffered in registers.
 //
 // The reference's recipe (src/gemm/ref/Kernels.cpp:412-747: global prefetch ahead of use, LDS multi-buffer,
 // LDS->register prefetch of the next k step while the current one is multiplied) mapped onto CDNA4:
 //   - global -> LDS: global_load_lds_dwordx4; no register staging, no LDS write instructions.  Each lane
-//     fetches the 16-byte chunk whose XOR-swizzled LDS slot is (wave, instruction, lane); the swizzle
-//     removes the bank conflicts that padding would (a direct load writes 1 KB contiguously, so rows
-//     cannot be padded).
-//   - measured on MI355X, a 64 KB batch of such loads takes about 3,000 clocks to land when all 256 CUs
-//     stream (most requests hit in L2 but wait on lines a neighbour's miss is still fetching), while one
-//     slice is multiplied in about 1,000.  The ring therefore keeps four slices (128 KB) in flight per CU and
-//     gives each batch three slice times to land: 5 x 32 KB = all 160 KB of LDS.
-//   - each wavefront issues the LDS fragment reads of slice s+1 into its second register set, then the 16
-//     MFMAs of slice s from the first; one barrier per slice hands buffers over.
+//     fetches the 16-byte chunk whose XOR-swizzled LDS slot is (wave, instruction, lane); the swizzle removes
+//     the bank conflicts that padding would (a direct load writes 1 KB contiguously, so rows cannot be padded).
+//   - measured on MI355X, a batch of direct loads takes about 3,000 clocks to land when all 256 CUs stream,
+//     while a 256 x 256 fp16 slice is multiplied in about 1,000: the ring keeps DEPTH-1 slices in flight per
+//     work-group and gives each batch DEPTH-2 slice times to land.
+//   - each wavefront issues its share of slice s+DEPTH, then the MFMAs of slice s from one register set with
+//     the LDS fragment reads of slice s+1 (into the other set) spread between them, then one barrier.
 #pragma once
 
 #include <type_traits>
@@ -27,36 +25,9 @@ namespace mmbo {
 
 namespace ring {
 
-constexpr int BM = 256, BN = 256, BK = 32, NT = 512;
-constexpr int DEPTH = 5;                         // ring buffers
-constexpr int TILE_BYTES = 256 * BK * 2;         // one operand tile of one slice: 16 KB
-constexpr int SLICE_BYTES = 2 * TILE_BYTES;      // A then B: 32 KB
-constexpr int LDS_BYTES = DEPTH * SLICE_BYTES;   // 160 KB
-constexpr int LOADS = 2;                         // direct loads per thread per operand per slice
-
-// ---- swizzled tile layouts (byte offsets inside a 16 KB operand tile) -------------------------------
-// KC (source contiguous along k): row r holds its 32 k values in 64 bytes = 4 chunks of 16 B; chunk c is
-//   stored at position c ^ ((r >> 2) & 3), so 16 consecutive rows reading the same logical chunk cover
-//   all sixteen 16-byte groups of the 256-byte-wide LDS.
-__device__ inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4); }
-// RC (source contiguous along the row index): k-row k holds 256 rows in 512 bytes = 32 chunks; chunk c is
-//   stored at c ^ ((k & 3) << 2): the four k-rows one transposing read touches land in different groups.
-__device__ inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * 512 + ((chunk ^ ((k & 3) << 2)) << 4); }
-
-// Global byte offset (from the tile origin of this slice) of the chunk thread (wave, lane) must fetch with
-// its i-th direct load so that it lands in LDS slot (wave*LOADS + i)*64 + lane.
-template <bool KC>
-__device__ inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld)
-{
-    if (KC) {
-        uint32_t row = (wave * LOADS + i) * 16 + (lane >> 2);
-        uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
-        return (row * ld + chunk * 8) * 2;
-    }
-    uint32_t k = (wave * LOADS + i) * 2 + (lane >> 5);
-    uint32_t chunk = (lane & 31) ^ ((k & 3) << 2);
-    return (k * ld + chunk * 8) * 2;
-}
+template <typename T> struct Slice;
+template <> struct Slice<half_t> { static constexpr int BK = 32; };
+template <> struct Slice<float>  { static constexpr int BK = 16; };
 
 template <int N, typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>)
@@ -66,12 +37,12 @@ __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F &&f)
 {
-    static_for_impl<N>(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
+    if constexpr (N > 0) static_for_impl<N>(static_cast<F &&>(f), std::make_integer_sequence<int, N>{});
 }
 
-// LDS reads are inline assembly with explicit s_waitcnt: the compiler cannot tell that a fragment read
-// never aliases an in-flight direct load (they target different ring buffers) and would otherwise drain
-// vmcnt before every read, which would serialise the ring.
+// LDS reads are inline assembly with explicit s_waitcnt: the compiler cannot tell that a fragment read never
+// aliases an in-flight direct load (they target different ring buffers) and would otherwise drain vmcnt
+// before every read, which would serialise the ring.
 template <int OFF>
 __device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr)
 {
@@ -86,16 +57,75 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr)
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
     return r;
 }
+template <int OFF>
+__device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr)
+{
+    uint32_t r;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+    return r;
+}
 
-// One operand of one wavefront for one slice: F row-blocks of 32 x 2 k-groups of 16, fetched by NOPS
-// separate LDS reads so the caller can spread them between MFMAs.
-template <bool KC, int F>
+// One operand tile of one slice: R rows x BK along k = R * 64 bytes, loaded by NW wavefronts.
+//   KC (source contiguous along k): LDS row r = its 64 bytes = 4 chunks of 16 B; chunk c sits at position
+//     c ^ ((r >> 2) & 3), so 16 consecutive rows reading the same logical chunk cover all sixteen 16-byte
+//     groups of the 256-byte-wide LDS.
+//   RC (source contiguous along the row index): LDS k-row = R elements; its chunks are XOR-swizzled with a
+//     mask that depends on k so that the k-rows one fragment read touches fall in different bank groups:
+//       fp16 (ds_read_b64_tr_b16 reads four consecutive k-rows x 32 B): mask from k & 3;
+//       fp32 (ds_read_b32: lanes 0-31 one k-row, lanes 32-63 the k-row four further): mask from (k >> 2) & 1.
+template <typename T, bool KC, int R, int NW>
+struct RingTile {
+    static constexpr int ESZ = sizeof(T);
+    static constexpr int BK = Slice<T>::BK;
+    static constexpr int BYTES = R * 64;
+    static constexpr int INSTRS = R / 16;                    // direct-load instructions (1 KB each) per slice
+    static_assert(INSTRS % NW == 0, "tile must split evenly over the wavefronts");
+    static constexpr int LPW = INSTRS / NW;                  // loads per thread per slice
+    static constexpr int ROW_BYTES = R * ESZ;                // RC: one k-row
+    static constexpr int CPR = ROW_BYTES / 16;               // RC: chunks per k-row
+    static constexpr int KPI = 1024 / ROW_BYTES;             // RC: k-rows per load instruction
+    static_assert(KC || (ROW_BYTES <= 1024 && 1024 % ROW_BYTES == 0 && CPR >= (ESZ == 4 ? 16 : 8)),
+                  "RC tile: a k-row must be 128 (fp16) or 256 .. 1024 bytes, a power of two");
+
+    __device__ static inline uint32_t rc_mask(uint32_t k)
+    {
+        if constexpr (ESZ == 4) return ((k >> 2) & 1) << 3;                  // shift by 128 B
+        else if constexpr (ROW_BYTES % 256 == 0) return (k & 3) << 2;        // shift by 64 B per k
+        else if constexpr (ROW_BYTES % 256 == 128) return ((k >> 1) & 1) << 2;
+        else return 0;
+    }
+    __device__ static inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4); }
+    __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4); }
+
+    // Global byte offset (from the tile origin of this slice) of the chunk thread (wave, lane) must fetch with
+    // its i-th direct load so that it lands in LDS slot (wave*LPW + i)*64 + lane.
+    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld)
+    {
+        const uint32_t q = wave * LPW + i;
+        if constexpr (KC) {
+            uint32_t row = q * 16 + (lane >> 2);
+            uint32_t chunk = (lane & 3) ^ ((row >> 2) & 3);
+            return row * ld * ESZ + chunk * 16;
+        } else {
+            uint32_t k = q * KPI + lane / CPR;
+            uint32_t chunk = (lane % CPR) ^ rc_mask(k);
+            return k * ld * ESZ + chunk * 16;
+        }
+    }
+};
+
+// Fragments of one operand of one wavefront for one slice: F row-blocks of 32 x 2 k-groups.  A k-group is what one
+// 128-bit register quad per lane feeds: 16 k values (one 32x32x16 f16 MFMA) or 8 (four 32x32x2 f32 MFMAs).
+// Lane group g = lane/32, element e holds k = kg*KG + g*VEC + e, for both operands alike.
+template <typename T, bool KC, int R, int NW, int F>
 struct SliceFrags {
-    static constexpr int NOPS = KC ? 2 * F : 4 * F;
-    u32x4 x[2][KC ? F : 1];          // KC: one 128-bit read per fragment
-    u32x2 y[2][KC ? 1 : F][2];       // RC: two transposing 64-bit reads per fragment
+    using Tile = RingTile<T, KC, R, NW>;
+    static constexpr int ESZ = sizeof(T);
+    static constexpr int RPF = KC ? 1 : (ESZ == 2 ? 2 : 4);     // LDS reads per fragment
+    static constexpr int NOPS = 2 * F * RPF;
+    u32x4 x[2][F];
 
-    struct Addr { uint32_t a[KC ? 2 : F]; };      // per-lane byte offsets inside the operand tile
+    struct Addr { uint32_t a[KC ? 2 : F]; };                    // per-lane byte offsets inside the operand tile
 
     __device__ static inline Addr make_addr(int lane, int r0)
     {
@@ -103,16 +133,24 @@ struct SliceFrags {
         if constexpr (KC) {
             uint32_t r = lane & 31, g = lane >> 5;
 #pragma unroll
-            for (int kg = 0; kg < 2; ++kg) ad.a[kg] = kc_off(r0 + r, kg * 2 + g);      // + f*32*64 per block
-        } else {
-            // transposing read: lane j of a 16-lane block points at k-row j/4, rows 4*(j%4)..+3, and
-            // receives (k-rows 0..3) x (row j)
+            for (int kg = 0; kg < 2; ++kg) ad.a[kg] = Tile::kc_off(r0 + r, kg * 2 + g);   // + f*32*64 per block
+        } else if constexpr (ESZ == 2) {
+            // transposing read: lane j of a 16-lane block points at k-row j/4, rows 4*(j%4)..+3, and receives
+            // (k-rows 0..3) x (row j)
             uint32_t j = lane & 15, blk = (lane >> 4) & 1, g = lane >> 5;
 #pragma unroll
             for (int f = 0; f < F; ++f) {
                 uint32_t m = r0 + f * 32 + blk * 16 + (j & 3) * 4;
-                uint32_t k = g * 8 + (j >> 2);                                         // + kg*16 + h*4
-                ad.a[f] = rc_off(k, m >> 3) + (m & 7) * 2;
+                uint32_t k = g * 8 + (j >> 2);                                           // + kg*16 + h*4
+                ad.a[f] = Tile::rc_off(k, m >> 3) + (m & 7) * 2;
+            }
+        } else {
+            uint32_t r = lane & 31, g = lane >> 5;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                uint32_t m = r0 + f * 32 + r;
+                uint32_t k = g * 4;                                                      // + kg*8 + t
+                ad.a[f] = Tile::rc_off(k, m >> 2) + (m & 3) * 4;
             }
         }
         return ad;
@@ -122,42 +160,58 @@ struct SliceFrags {
     template <int OP>
     __device__ __forceinline__ void read_op(uint32_t tile, const Addr &ad)
     {
+        constexpr int kg = OP / (F * RPF), f = (OP / RPF) % F, h = OP % RPF;
         if constexpr (KC) {
-            constexpr int kg = OP / F, f = OP % F;
             x[kg][f] = lds_read_b128<f * 32 * 64>(tile + ad.a[kg]);
+        } else if constexpr (ESZ == 2) {
+            u32x2 v = lds_read_tr16_b64<(kg * 16 + h * 4) * Tile::ROW_BYTES>(tile + ad.a[f]);
+            x[kg][f][2 * h] = v[0];
+            x[kg][f][2 * h + 1] = v[1];
         } else {
-            constexpr int kg = OP / (2 * F), f = (OP / 2) % F, h = OP % 2;
-            y[kg][f][h] = lds_read_tr16_b64<kg * 16 * 512 + h * 4 * 512>(tile + ad.a[f]);
+            x[kg][f][h] = lds_read_b32<(kg * 8 + h) * Tile::ROW_BYTES>(tile + ad.a[f]);
         }
     }
     __device__ __forceinline__ void read_all(uint32_t tile, const Addr &ad)
     {
         static_for<NOPS>([&](auto OP) { this->template read_op<decltype(OP)::value>(tile, ad); });
     }
-    __device__ __forceinline__ f16x8 get(int kg, int f) const
-    {
-        if constexpr (KC) return __builtin_bit_cast(f16x8, x[kg][f]);
-        else return __builtin_bit_cast(f16x8, u32x4{y[kg][f][0][0], y[kg][f][0][1], y[kg][f][1][0], y[kg][f][1][1]});
-    }
 };
 
 }  // namespace ring
 
-// WM x WN wavefronts; wave tile (256/WM) x (256/WN).  WM*WN == 8.
 // ABLATE is a timing probe in the spirit of the reference's error_kernel_000.s / test_main_loop.s (kernels
 // with parts removed to find the ceiling of what is left; results are wrong by design): bit 0 drops the
 // global->LDS loads, bit 1 the LDS fragment reads, bit 2 the MFMAs, bit 3 writes the main loop's clock64 and
-// wall_clock64 spans to args.ws, bit 6 makes every work-group read the same tiles.  The library only instantiates ABLATE = 0.
-template <bool TA, bool TB, int WM, int WN, int ABLATE = 0>
-__global__ void __launch_bounds__(512)
-hgemm_ring_kernel(const GemmArgs args)
+// wall_clock64 spans to args.ws.  The library only instantiates ABLATE = 0.
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+struct RingCfg {
+    static constexpr int NW = WM * WN, NT = NW * 64;
+    static constexpr int BK = ring::Slice<T>::BK;
+    static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+    static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
+    using TileA = ring::RingTile<T, TA, BM, NW>;       // A is k-contiguous when transposed
+    using TileB = ring::RingTile<T, !TB, BN, NW>;      // B is k-contiguous when not transposed
+    using FragA = ring::SliceFrags<T, TA, BM, NW, FM>;
+    using FragB = ring::SliceFrags<T, !TB, BN, NW, FN>;
+    static constexpr int SLICE_BYTES = TileA::BYTES + TileB::BYTES;
+    static constexpr int LDS_BYTES = DEPTH * SLICE_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "ring does not fit the 160 KB of LDS");
+    static constexpr int BATCH = TileA::LPW + TileB::LPW;      // direct loads per thread per slice
+    static constexpr int MPK = sizeof(T) == 2 ? 1 : 4;         // MFMAs per (k-group, block pair)
+    static constexpr int NMFMA = 2 * FM * FN * MPK;
+};
+
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_ring_kernel(const GemmArgs args)
 {
     using namespace ring;
-    static_assert(WM * WN == 8, "eight wavefronts");
-    constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
-    constexpr bool A_KC = TA, B_KC = !TB;
-    using FragA = SliceFrags<A_KC, FM>;
-    using FragB = SliceFrags<B_KC, FN>;
+    using Cfg = RingCfg<T, TA, TB, BM, BN, WM, WN, DEPTH, ABLATE>;
+    using TileA = typename Cfg::TileA;
+    using TileB = typename Cfg::TileB;
+    using FragA = typename Cfg::FragA;
+    using FragB = typename Cfg::FragB;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, ESZ = sizeof(T), BATCH = Cfg::BATCH;
 
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -168,61 +222,59 @@ hgemm_ring_kernel(const GemmArgs args)
 
     uint32_t wg0, wg1;
     wg_remap(blockIdx.x, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
-    if constexpr (ABLATE & 64) { wg0 = 0; wg1 = 0; }          // probe: every work-group reads the same tiles
-    const uint32_t batch = blockIdx.z;
+    const uint32_t zb = blockIdx.z;
+    const uint32_t split = zb / args.batch, batch = zb % args.batch;
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
     const uint32_t lda = args.lda, ldb = args.ldb;
-    const int n_slice = (int)(args.k / BK);
+    const uint32_t k_begin = split * args.k_per_split;
+    const uint32_t k_end = min(args.k, k_begin + args.k_per_split);
+    const int n_slice = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
 
     const char *gA = static_cast<const char *>(args.A) +
-                     ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda : (int64_t)row0)) * 2;
+                     ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda + k_begin
+                                                          : (int64_t)k_begin * lda + row0)) * ESZ;
     const char *gB = static_cast<const char *>(args.B) +
-                     ((int64_t)batch * args.strideB + (TB ? (int64_t)col0 : (int64_t)col0 * ldb)) * 2;
-    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * 2;
-    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * 2;
+                     ((int64_t)batch * args.strideB + (TB ? (int64_t)k_begin * ldb + col0
+                                                          : (int64_t)col0 * ldb + k_begin)) * ESZ;
+    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * ESZ;
+    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * ESZ;
 
-    uint32_t offA[LOADS], offB[LOADS];
+    uint32_t offA[TileA::LPW], offB[TileB::LPW];
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        offA[i] = load_goff<A_KC>(wave, lane, i, lda);
-        offB[i] = load_goff<B_KC>(wave, lane, i, ldb);
-    }
+    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda);
+#pragma unroll
+    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb);
+
     // slice s goes to ring buffer s % DEPTH; `buf` is that index, kept by the caller
     auto issue_slice = [&](int s, int buf) {
         if constexpr (ABLATE & 1) return;
-        char *dst = lds + buf * SLICE_BYTES;
+        char *dst = lds + buf * Cfg::SLICE_BYTES;
         const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i)
+        for (int i = 0; i < TileA::LPW; ++i)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pa + offA[i]),
-                                             MMBO_LDS_PTR(dst + (wave * LOADS + i) * 1024), 16, 0, 0);
+                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + i) * 1024), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i)
+        for (int i = 0; i < TileB::LPW; ++i)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pb + offB[i]),
-                                             MMBO_LDS_PTR(dst + TILE_BYTES + (wave * LOADS + i) * 1024), 16, 0, 0);
+                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024), 16, 0, 0);
     };
-    constexpr int BATCH = 2 * LOADS;             // direct loads per thread per slice
 
-    const typename FragA::Addr adA = FragA::make_addr(lane, wm * TM);
-    const typename FragB::Addr adB = FragB::make_addr(lane, wn * TN);
+    const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
+    const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
     FragA fa[2];
     FragB fb[2];
     if constexpr (ABLATE != 0) {      // keep the probes' registers defined
+        const uint32_t va = (ESZ == 2 ? 0x3c003c00u : 0x3f800000u) + (uint32_t)lane;
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            const uint32_t va = 0x3c003c00u + (uint32_t)lane, vb = 0x38003800u + (uint32_t)lane;
+        for (int q = 0; q < 2; ++q)
 #pragma unroll
             for (int kg = 0; kg < 2; ++kg) {
 #pragma unroll
-                for (int f = 0; f < (A_KC ? FM : 1); ++f) fa[q].x[kg][f] = u32x4{va, va, va, va};
+                for (int f = 0; f < FM; ++f) fa[q].x[kg][f] = u32x4{va, va, va, va};
 #pragma unroll
-                for (int f = 0; f < (A_KC ? 1 : FM); ++f) fa[q].y[kg][f][0] = fa[q].y[kg][f][1] = u32x2{va, va};
-#pragma unroll
-                for (int f = 0; f < (B_KC ? FN : 1); ++f) fb[q].x[kg][f] = u32x4{vb, vb, vb, vb};
-#pragma unroll
-                for (int f = 0; f < (B_KC ? 1 : FN); ++f) fb[q].y[kg][f][0] = fb[q].y[kg][f][1] = u32x2{vb, vb};
+                for (int f = 0; f < FN; ++f) fb[q].x[kg][f] = u32x4{va, va, va, va};
             }
-        }
     }
 
     f32x16 acc[FM][FN];
@@ -236,28 +288,38 @@ hgemm_ring_kernel(const GemmArgs args)
     const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         if constexpr (ABLATE & 2) return;
-        const uint32_t t = lds_base + buf * SLICE_BYTES;
+        const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
-        b.read_all(t + TILE_BYTES, adB);
+        b.read_all(t + TileA::BYTES, adB);
     };
-    // The 16 MFMAs of slice s with the LDS reads of slice s+1 spread between them.  Issued as one block, the
-    // reads of all eight wavefronts would fill the LDS queue and each wavefront would sit behind its own
-    // last read before reaching its first MFMA.
-    constexpr int NA = FragA::NOPS, NR = FragA::NOPS + FragB::NOPS, NMFMA = 2 * FM * FN;
+    // The MFMAs of slice s with the LDS reads of slice s+1 spread between them.  Issued as one block, the reads
+    // of all wavefronts would fill the LDS queue and each wavefront would sit behind its own last read before
+    // reaching its first MFMA.
+    constexpr int NA = FragA::NOPS, NR = FragA::NOPS + FragB::NOPS, NMFMA = Cfg::NMFMA, MPK = Cfg::MPK;
     auto mfma_and_read = [&](const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf) {
-        const uint32_t t = lds_base + nbuf * SLICE_BYTES;
+        const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
-            constexpr int kg = m / (FM * FN), i = (m / FN) % FM, j = m % FN;
-            if constexpr (!(ABLATE & 4))
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ca.get(kg, i), cb.get(kg, j), acc[i][j], 0, 0, 0);
+            // consecutive MFMAs go to different accumulators
+            constexpr int kg = m / (FM * FN * MPK), tt = (m / (FM * FN)) % MPK, i = (m / FN) % FM, j = m % FN;
+            if constexpr (!(ABLATE & 4)) {
+                if constexpr (ESZ == 2)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ca.x[kg][i]),
+                                                                       __builtin_bit_cast(f16x8, cb.x[kg][j]), acc[i][j], 0, 0, 0);
+                else {
+                    // (through locals: bit-casting a vector-element expression directly picked element 0)
+                    const uint32_t ua = ca.x[kg][i][tt], ub = cb.x[kg][j][tt];
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, ua),
+                                                                     __builtin_bit_cast(float, ub), acc[i][j], 0, 0, 0);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (!(ABLATE & 2)) {
                 constexpr int r0 = NR * m / NMFMA, r1 = NR * (m + 1) / NMFMA;
-                static_for<r1 - r0>([&](auto R) {
-                    constexpr int r = r0 + decltype(R)::value;
+                static_for<r1 - r0>([&](auto RR) {
+                    constexpr int r = r0 + decltype(RR)::value;
                     if constexpr (r < NA) na.template read_op<r>(t, adA);
-                    else nb.template read_op<r - NA>(t + TILE_BYTES, adB);
+                    else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -278,10 +340,10 @@ hgemm_ring_kernel(const GemmArgs args)
     // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
     // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free; this
     // wavefront's loads of slices s+2 .. s+DEPTH-1 are in flight.
-    //   iteration s:  issue loads(s+DEPTH) -> buffer s % DEPTH;  read slice s+1 -> set (s+1)&1;
-    //                 MFMAs of slice s from set s&1;  wait reads;  wait own loads(s+2);  barrier B_{s+1}.
-    // Loads return in order, so "all but the newest (DEPTH-2) batches" means loads(s+2) have landed; once
-    // the tail stops issuing, the wait is for everything.
+    //   iteration s:  issue loads(s+DEPTH) -> buffer s % DEPTH;  MFMAs of slice s from set s&1 interleaved with
+    //                 the reads of slice s+1 -> set (s+1)&1;  wait reads;  wait own loads(s+2);  barrier B_{s+1}.
+    // Loads return in order, so "all but the newest (DEPTH-2) batches" means loads(s+2) have landed; once the
+    // tail stops issuing, the wait is for everything.
 #pragma unroll
     for (int s = 0; s < DEPTH; ++s)
         if (s < n_slice) issue_slice(s, s);
@@ -311,7 +373,7 @@ hgemm_ring_kernel(const GemmArgs args)
         if (s + 1 < n_slice) step(s + 1, fa[1], fb[1], fa[0], fb[0]);
     }
     if constexpr (ABLATE & 8) {
-        if (tid == 0 && blockIdx.x == 300) {
+        if (tid == 0 && blockIdx.x == args.nwg0 * args.nwg1 / 3) {
             reinterpret_cast<long long *>(args.ws)[0] = clock64() - t_clk;
             reinterpret_cast<long long *>(args.ws)[1] = wall_clock64() - t_wall;
         }
@@ -320,45 +382,7 @@ hgemm_ring_kernel(const GemmArgs args)
 #undef MMBO_WAIT_VM
 #undef MMBO_WAIT_LGKM0
 
-    // ---- write-back: same accumulator layout as the staged kernel; every tile is interior here.
-    //   acc[i][j][4*q + r] is C(row0 + wm*TM + i*32 + 8*q + 4*(lane/32) + r,  col0 + wn*TN + j*32 + lane%32)
-    const float alpha = args.alpha, beta = args.beta;
-    const uint32_t ldc = args.ldc;
-    half_t *C = static_cast<half_t *>(args.C) + (int64_t)batch * args.strideC;
-    const int g = lane >> 5, cl = lane & 31;
-    const bool vec_c = args.vec_c != 0;
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            uint32_t col = col0 + wn * TN + j * 32 + cl;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t row = row0 + wm * TM + i * 32 + 8 * q + 4 * g;
-                half_t *p = C + (size_t)col * ldc + row;
-                float v[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * q + r];
-                if (vec_c) {
-                    union { half_t e[4]; u32x2 v2; } io;
-                    if (beta != 0.0f) {                       // beta == 0: C is never read
-                        io.v2 = *reinterpret_cast<const u32x2 *>(p);
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
-                    }
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) io.e[r] = (half_t)v[r];
-                    *reinterpret_cast<u32x2 *>(p) = io.v2;
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        float o = v[r];
-                        if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
-                        p[r] = (half_t)o;
-                    }
-                }
-            }
-        }
+    write_back<T, FM, FN, true>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, split, lane);
 }
 
 }  // namespace mmbo

@@ -272,72 +272,7 @@ gemm_staged_kernel(const GemmArgs args)
         cur ^= 1;
     }
 
-    // ---- write-back.  acc[i][j][4*q + r] is C(row, col) with
-    //   row = row0 + wm*TM + i*32 + 8*q + 4*(lane/32) + r,   col = col0 + wn*TN + j*32 + lane%32.
-    const uint32_t m = args.m, n = args.n;
-    const int g = lane >> 5, cl = lane & 31;
-    if (args.splits > 1) {
-        // partial sums, fp32, dense [split][batch][n][m]; alpha/beta are applied by the reduction
-        float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)m * n;
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                uint32_t col = col0 + wn * Cfg::TN + j * 32 + cl;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    uint32_t row = row0 + wm * Cfg::TM + i * 32 + 8 * q + 4 * g;
-                    if (col < n) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (row + r < m) ws[(size_t)col * m + row + r] = acc[i][j][4 * q + r];
-                    }
-                }
-            }
-        return;
-    }
-
-    const float alpha = args.alpha, beta = args.beta;
-    const uint32_t ldc = args.ldc;
-    T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
-    const bool vec_c = args.vec_c != 0;
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            uint32_t col = col0 + wn * Cfg::TN + j * 32 + cl;
-            if (col >= n) continue;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t row = row0 + wm * Cfg::TM + i * 32 + 8 * q + 4 * g;
-                if (row >= m) continue;
-                T *p = C + (size_t)col * ldc + row;
-                float v[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * q + r];
-                if (vec_c && row + 4 <= m) {
-                    union { T e[4]; u32x4 v4; u32x2 v2; } io;
-                    if (beta != 0.0f) {                       // beta == 0: C is never read
-                        if constexpr (ESZ == 4) io.v4 = *reinterpret_cast<const u32x4 *>(p);
-                        else io.v2 = *reinterpret_cast<const u32x2 *>(p);
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
-                    }
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) io.e[r] = (T)v[r];
-                    if constexpr (ESZ == 4) *reinterpret_cast<u32x4 *>(p) = io.v4;
-                    else *reinterpret_cast<u32x2 *>(p) = io.v2;
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (row + r < m) {
-                            float o = v[r];
-                            if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
-                            p[r] = (T)o;
-                        }
-                }
-            }
-        }
+    write_back<T, FM, FN, false>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, split, lane);
 }
 
 // Split-K reduction: C = alpha * sum_s ws[s] + beta * C, splits added in ascending order so the

@@ -1,38 +1,49 @@
-// Instantiates the HGEMM ring kernel for the four transpose pairs.
+// Instantiates the ring kernel for one (element type, ring tile row): compile with
+//   -DMMBO_DTYPE=<0|1> -DMMBO_TILE=<row>
+#include "configs.hpp"
 #include "gemm_ring.hpp"
 #include "launch.hpp"
+
+#ifndef MMBO_DTYPE
+#error "MMBO_DTYPE and MMBO_TILE select what this translation unit instantiates"
+#endif
 
 namespace mmbo {
 
 namespace {
+using ElemT = typename std::conditional<MMBO_DTYPE == 0, float, half_t>::type;
+constexpr RingRow R = kRingTiles[MMBO_TILE];
+
 template <bool TA, bool TB, int WM, int WN>
 hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
-    auto kernel = hgemm_ring_kernel<TA, TB, WM, WN>;
+    using Cfg = RingCfg<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
+    auto kernel = gemm_ring_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
     static bool attr_set[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64 && !attr_set[dev]) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                ring::LDS_BYTES);
+                                Cfg::LDS_BYTES);
         if (e != hipSuccess) return e;
         attr_set[dev] = true;
     }
-    dim3 grid(args.nwg0 * args.nwg1, 1, args.batch);
-    hipLaunchKernelGGL(kernel, grid, dim3(ring::NT), ring::LDS_BYTES, stream, args);
+    dim3 grid(args.nwg0 * args.nwg1, 1, args.batch * args.splits);
+    hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
 }  // namespace
 
-// Wave layout per transpose pair: the operand that needs transposing LDS reads (two reads per fragment)
-// gets the fewer fragments.
-hipError_t launch_hgemm_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream)
+// Wave layout per transpose pair: the operand that needs transposing LDS reads (two or four reads per fragment
+// instead of one) gets the fewer fragments.  A needs them under transA = N, B under transB = T.
+template <>
+hipError_t launch_ring<MMBO_DTYPE, MMBO_TILE>(int transA, int transB, const GemmArgs &args, hipStream_t stream)
 {
-    if (!transA && !transB) return launch_one<false, false, 4, 2>(args, stream);
-    if (!transA && transB) return launch_one<false, true, 4, 2>(args, stream);
-    if (transA && !transB) return launch_one<true, false, 4, 2>(args, stream);
-    return launch_one<true, true, 2, 4>(args, stream);
+    if (!transA && !transB) return launch_one<false, false, R.wm, R.wn>(args, stream);
+    if (!transA && transB) return launch_one<false, true, R.wm, R.wn>(args, stream);
+    if (transA && !transB) return launch_one<true, false, R.wm, R.wn>(args, stream);
+    return launch_one<true, true, R.wn, R.wm>(args, stream);
 }
 
 }  // namespace mmbo

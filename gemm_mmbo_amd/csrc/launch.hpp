@@ -15,6 +15,10 @@ hipError_t launch_staged(int transA, int transB, const GemmArgs &args, hipStream
 template <int DTYPE, int TILE>
 int staged_lds_bytes();
 
+// Ring kernel of ring tile row TILE; grid = (nwg0*nwg1, 1, batch*splits).
+template <int DTYPE, int TILE>
+hipError_t launch_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream);
+
 hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream);
 
 }  // namespace mmbo

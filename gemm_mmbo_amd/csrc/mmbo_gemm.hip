@@ -15,19 +15,34 @@
 
 namespace mmbo {
 
-hipError_t launch_hgemm_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream);
-
 namespace {
 
-// Config ids: [0, NUM_TILES*NUM_SPLITS) are the staged kernel's (tile, split) pairs; fp16 has one more,
-// the direct-to-LDS ring kernel, usable when m, n are multiples of 256, k of 32 and operands aligned.
+// Config ids: [0, kStagedConfigs) are the staged kernel's (tile, split) pairs, then the ring kernel's
+// (ring tile, split) pairs.  A ring config applies when m, n are multiples of its tile, k splits into whole
+// slices and A, B are 16-byte aligned; otherwise the call is refused with MMBO_ERR_INVALID_CONFIG.
 constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
-constexpr int kRingConfig = kStagedConfigs;
-inline int num_configs_of(int dtype) { return dtype == MMBO_F16 ? kStagedConfigs + 1 : kStagedConfigs; }
+constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
+constexpr int kNumConfigs = kStagedConfigs + kRingConfigs;
 
-inline bool ring_eligible(int dtype, size_t m, size_t n, size_t k)
+struct ConfigRef {
+    bool ring;
+    int tile;
+    int split;
+};
+inline ConfigRef config_ref(int id)
 {
-    return dtype == MMBO_F16 && m % 256 == 0 && n % 256 == 0 && k % 32 == 0 && k >= 32;
+    if (id < kStagedConfigs) return {false, id % NUM_TILES, kSplits[id / NUM_TILES]};
+    id -= kStagedConfigs;
+    return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES]};
+}
+inline int ring_config_id(int tile, int split_index) { return kStagedConfigs + tile + NUM_RING_TILES * split_index; }
+
+inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k)
+{
+    const RingRow &r = kRingTiles[tile];
+    const size_t bk = (size_t)ring_bk(dtype);
+    if (m % r.bm || n % r.bn || k == 0 || k % bk) return false;
+    return (k / bk) % (size_t)split == 0;          // every split gets the same whole number of slices
 }
 
 thread_local int g_last_hip_error = 0;
@@ -82,6 +97,14 @@ hipError_t dispatch_tile(int tile, int ta, int tb, const GemmArgs &a, hipStream_
 {
     if (tile == TILE) return launch_staged<DTYPE, TILE>(ta, tb, a, s);
     if constexpr (TILE + 1 < NUM_TILES) return dispatch_tile<DTYPE, TILE + 1>(tile, ta, tb, a, s);
+    return hipErrorInvalidValue;
+}
+
+template <int DTYPE, int TILE>
+hipError_t dispatch_ring(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
+{
+    if (tile == TILE) return launch_ring<DTYPE, TILE>(ta, tb, a, s);
+    if constexpr (TILE + 1 < NUM_RING_TILES) return dispatch_ring<DTYPE, TILE + 1>(tile, ta, tb, a, s);
     return hipErrorInvalidValue;
 }
 
@@ -179,19 +202,28 @@ const char *mmbo_status_string(int status)
 int mmbo_num_configs(int dtype)
 {
     if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
-    return num_configs_of(dtype);
+    return kNumConfigs;
 }
 
 int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
 {
     if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
     if (!out) return MMBO_ERR_NULL_POINTER;
-    if (config_id < 0 || config_id >= num_configs_of(dtype)) return MMBO_ERR_INVALID_CONFIG;
+    if (config_id < 0 || config_id >= kNumConfigs) return MMBO_ERR_INVALID_CONFIG;
     std::memset(out, 0, sizeof(*out));
-    if (config_id == kRingConfig) {
-        std::snprintf(out->name, sizeof(out->name), "MT256x256x32_WT064x128_W8_GSU01_DTL1_RING5");
-        out->macro_tile_m = 256; out->macro_tile_n = 256; out->depth_u = 32; out->threads = 512;
-        out->wave_tile_m = 64; out->wave_tile_n = 128; out->split_k = 1; out->lds_bytes = 160 * 1024;
+    const ConfigRef c = config_ref(config_id);
+    if (c.ring) {
+        const RingRow &r = kRingTiles[c.tile];
+        std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d", r.bm, r.bn,
+                      ring_bk(dtype), r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, c.split, r.depth);
+        out->macro_tile_m = r.bm;
+        out->macro_tile_n = r.bn;
+        out->depth_u = ring_bk(dtype);
+        out->threads = r.wm * r.wn * 64;
+        out->wave_tile_m = r.bm / r.wm;
+        out->wave_tile_n = r.bn / r.wn;
+        out->split_k = c.split;
+        out->lds_bytes = r.depth * (r.bm + r.bn) * 64;
         return MMBO_OK;
     }
     int tile = config_id % NUM_TILES, split = kSplits[config_id / NUM_TILES];
@@ -230,9 +262,18 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
             if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
         }
     }
-    // the ring kernel replaces the big staged tiles wherever it applies
-    // the ring kernel replaces the big staged tiles wherever it applies
-    if (ring_eligible(dtype, m, n, k) && best < NUM_TILES && best <= 1) best = kRingConfig;
+    // ring configs: same tile geometry, deeper prefetch, no edge handling.  Where one applies it replaces the
+    // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).
+    {
+        const ConfigRef c = config_ref(best);
+        const TileRow &t = tile_row(dtype, c.tile);
+        for (int rt = 0; rt < NUM_RING_TILES; ++rt) {
+            const RingRow &r = kRingTiles[rt];
+            if (r.bm * r.bn > t.bm * t.bn) continue;
+            for (int si = 0; si < NUM_SPLITS; ++si)
+                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k)) return ring_config_id(rt, si);
+        }
+    }
     return best;
 }
 
@@ -286,7 +327,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
             return MMBO_ERR_INVALID_SIZE;
     }
     if (strideA < 0 || strideB < 0 || strideC < 0) return MMBO_ERR_INVALID_SIZE;
-    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= num_configs_of(dtype)))
+    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= kNumConfigs))
         return MMBO_ERR_INVALID_CONFIG;
     if (m == 0 || n == 0 || batch == 0) return MMBO_OK;          // nothing to write
     if (!C) return MMBO_ERR_NULL_POINTER;
@@ -299,12 +340,12 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
     }
-    const bool use_ring = config_id == kRingConfig;
-    if (use_ring) config_id = 0;                                // same macro tile as staged row 0, no split
-    int tile = config_id % NUM_TILES;
-    int split = kSplits[config_id / NUM_TILES];
-    const TileRow &r = tile_row(dtype, tile);
+    const ConfigRef cref = config_ref(config_id);
     const size_t esz = dtype == MMBO_F32 ? 4 : 2;
+    int split = cref.split;
+    TileRow r = cref.ring ? TileRow{kRingTiles[cref.tile].bm, kRingTiles[cref.tile].bn, ring_bk(dtype), 0, 0}
+                          : tile_row(dtype, cref.tile);
+    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
     // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
     {
@@ -344,18 +385,17 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     a.vec_c = aligned16(C, ldc, strideC);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (use_ring) {
-        if (!ring_eligible(dtype, m, n, k) || !a.vec_a || !a.vec_b) return MMBO_ERR_INVALID_CONFIG;
-        hipError_t e = launch_hgemm_ring(transA, transB, a, s);
-        return e == hipSuccess ? MMBO_OK : hip_fail(e);
-    }
+    if (cref.ring && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
     if (split > 1) {
         size_t bytes = (size_t)split * batch * m * n * sizeof(float);
         int rc = workspace(bytes, &a.ws);
         if (rc != MMBO_OK) return rc;
     }
-    hipError_t e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(tile, transA, transB, a, s)
-                                     : dispatch_tile<1, 0>(tile, transA, transB, a, s);
+    hipError_t e;
+    if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
+                                         : dispatch_ring<1, 0>(cref.tile, transA, transB, a, s);
+    else e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(cref.tile, transA, transB, a, s)
+                               : dispatch_tile<1, 0>(cref.tile, transA, transB, a, s);
     if (e != hipSuccess) return hip_fail(e);
     if (split > 1) {
         e = launch_splitk_reduce(dtype, a, s);

@@ -17,22 +17,24 @@ struct TunedRow {
 };
 
 constexpr TunedRow kTuned[] = {
-    //dtype ta tb     m      n      k  batch  id   TFLOP/s
-    {0, 0, 0,  1024,  1024,  1024,  1,   4,   77.8f},
-    {0, 0, 1,  4096,  4096,  4096,  1,   0,  131.3f},
-    {0, 1, 0,  4096,  4096,  4096,  1,   0,  127.2f},
-    {0, 0, 0,  8192,  8192,  8192,  1,   0,  137.0f},
-    {1, 0, 0,  8192,  8192,  8192,  1,  30, 1020.0f},
-    {0, 0, 0,  1023,   777,   513,  1,   4,   24.7f},
-    {1, 0, 0,  1023,   777,   513,  1,  16,   26.3f},
-    {0, 0, 0,  4096,   128,  4096,  1,  22,   79.5f},
-    {1, 0, 0,  4096,   128,  4096,  1,  16,  192.6f},
-    {0, 0, 0,   128,  4096,  8192,  1,  21,   94.1f},
-    {1, 0, 0,   128,  4096,  8192,  1,  16,  281.6f},
-    {1, 1, 0,   512,   512,   512, 64,  30,  412.4f},
-    {0, 0, 0,  2048,  2048,  2048,  1,   3,  113.8f},
-    {1, 0, 0,  2048,  2048,  2048,  1,   3,  559.6f},
-    {0, 0, 1, 44160,  2048,   384,  1,   3,  114.1f},
+    //dtype ta tb m n k batch id TFLOP/s
+    {0, 0, 0, 1024, 1024, 1024, 1, 4, 75.4f},
+    {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
+    {0, 1, 0, 4096, 4096, 4096, 1, 30, 137.1f},
+    {0, 0, 0, 1023, 777, 513, 1, 10, 24.5f},
+    {1, 0, 0, 1023, 777, 513, 1, 16, 26.3f},
+    {0, 0, 0, 4096, 128, 4096, 1, 22, 85.8f},
+    {1, 0, 0, 4096, 128, 4096, 1, 41, 232.0f},
+    {0, 0, 0, 128, 4096, 8192, 1, 47, 100.1f},
+    {1, 0, 0, 128, 4096, 8192, 1, 41, 325.0f},
+    {1, 1, 0, 512, 512, 512, 64, 30, 402.1f},
+    {0, 0, 0, 2048, 2048, 2048, 1, 3, 112.0f},
+    {1, 0, 0, 2048, 2048, 2048, 1, 3, 557.1f},
+    {0, 0, 1, 44160, 2048, 384, 1, 2, 107.1f},
+    {0, 0, 0, 8192, 8192, 8192, 1, 30, 142.0f},
+    {1, 0, 0, 8192, 8192, 8192, 1, 30, 1075.9f},
+    {0, 0, 0, 4096, 4096, 4096, 1, 30, 140.6f},
+    {1, 0, 0, 4096, 4096, 4096, 1, 30, 1018.2f},
 };
 
 }  // namespace mmbo

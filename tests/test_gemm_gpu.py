@@ -94,23 +94,52 @@ def test_every_config_aligned_interior(dtype):
         _run_and_check(p, cid, label=f"config {cid}")
 
 
+def _ring_ids(dtype):
+    import gemm_mmbo_amd as G
+    return [c for c in range(G.num_configs(dtype)) if "DTL1" in G.config_info(dtype, c)["name"]]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
-def test_direct_to_lds_ring_kernel_every_transpose(ta, tb):
-    """The HGEMM fast path (global->LDS direct loads through a five-deep ring) by explicit config id: short and
-    long K (fewer slices than ring buffers, odd slice counts), beta read-modify-write, ld > dim, batches."""
+def test_ring_kernel_every_config_every_transpose(dtype, ta, tb):
+    """The direct-to-LDS ring kernel by explicit config id: every ring tile and split-K factor, with K shorter
+    and longer than the ring (fewer slices than buffers, odd slice counts), beta read-modify-write, batches."""
     import gemm_mmbo_amd as G
-    cid = G.num_configs(F16) - 1
-    assert "DTL1" in G.config_info(F16, cid)["name"]
-    for (m, n, k, alpha, beta, batch) in ((256, 256, 32, 1.0, 0.0, 1), (512, 256, 96, 1.5, 0.5, 1), (256, 768, 160, 1.0, 0.0, 1),
-                                          (768, 1024, 1056, -1.0, 1.0, 1), (256, 512, 4096, 1.0, 0.0, 1), (256, 256, 224, 1.0, 1.0, 3)):
-        p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=70 + k, dist="normal",
-                      c_fill="uniform" if beta else "nan")
-        _run_and_check(p, cid, label=f"ring {m}x{n}x{k} b{batch}")
-    p = U.Problem(F16, ta, tb, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71, dist="normal")
+    ids = _ring_ids(dtype)
+    assert len(ids) == 20
+    bk = 16 if dtype == F32 else 32
+    ran = 0
+    for cid in ids:
+        d = G.config_info(dtype, cid)
+        bm, bn, sp = d["macro_tile_m"], d["macro_tile_n"], d["split_k"]
+        for (tm, tn, slices, alpha, beta, batch) in ((1, 1, 1, 1.0, 0.0, 1), (2, 1, 3, 1.5, 0.5, 1), (1, 3, 7, -1.0, 1.0, 2),
+                                                     (3, 2, 33, 1.0, 0.0, 1)):
+            m, n, k = bm * tm, bn * tn, bk * slices * sp
+            p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, batch=batch, seed=70 + cid + slices,
+                          dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
+            _run_and_check(p, cid, label=f"{d['name']} {m}x{n}x{k} b{batch}")
+            ran += 1
+    assert ran == 80
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_ring_kernel_refuses_shapes_it_cannot_take(dtype):
+    """Ragged m/n, k that does not split into whole slices, unaligned A: MMBO_ERR_INVALID_CONFIG, never a wrong
+    result; the automatic pick falls back to the staged kernel and still matches the oracle."""
+    import gemm_mmbo_amd as G
+    cid = _ring_ids(dtype)[0]
+    bk = 16 if dtype == F32 else 32
+    for (m, n, k, offs) in ((255, 256, 4 * bk, (0, 0, 0)), (256, 300, 4 * bk, (0, 0, 0)), (256, 256, 4 * bk + 8, (0, 0, 0)),
+                            (256, 256, 4 * bk, (1, 0, 0))):
+        p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
+        with pytest.raises(G.MmboError) as e:
+            U.run_gpu(p, cid, offs)
+        assert e.value.status == 5
+        _run_and_check(p, -1, label="auto fallback", offsets=offs)
+    p = U.Problem(dtype, 1, 0, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71)
     _run_and_check(p, cid, label="ring ld>dim")
-    # the per-shape table picks it for the headline shape
-    assert G.select_config(F16, ta, tb, 8192, 8192, 8192) == cid
+    assert "DTL1" in G.config_info(dtype, G.select_config(dtype, 0, 0, 8192, 8192, 8192))["name"]
 
 
 # ------------------------------------------------------------------ edges
