@@ -292,12 +292,16 @@ gemm_ring_kernel(const GemmArgs args)
         a.read_all(t, adA);
         b.read_all(t + TileA::BYTES, adB);
     };
-    // The MFMAs of slice s with the LDS reads of slice s+1 spread between them.  Issued as one block, the reads
-    // of all wavefronts would fill the LDS queue and each wavefront would sit behind its own last read before
-    // reaching its first MFMA.
+    // The MFMAs of slice s with the LDS reads of slice s+1 and the direct loads of slice s+DEPTH spread between
+    // them.  A wavefront issues in order: issued as one block at the top of the slice, the reads of all
+    // wavefronts fill the LDS queue and the loads the texture-address queue, and every wavefront sits behind
+    // its own last memory instruction before it reaches its first MFMA (measured: ~300 clocks per slice lost to
+    // the reads, ~450 to the loads).
     constexpr int NA = FragA::NOPS, NR = FragA::NOPS + FragB::NOPS, NMFMA = Cfg::NMFMA, MPK = Cfg::MPK;
-    auto mfma_and_read = [&](const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf) {
+    auto mfma_and_read = [&](const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
+        char *dst = lds + lbuf * Cfg::SLICE_BYTES;
+        const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // consecutive MFMAs go to different accumulators
@@ -322,6 +326,25 @@ gemm_ring_kernel(const GemmArgs args)
                     else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
+            if constexpr (!(ABLATE & 1)) {
+                // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
+                constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
+                static_for<l1 - l0>([&](auto LL) {
+                    constexpr int l = l0 + decltype(LL)::value;
+                    if constexpr (l < BATCH) {
+                        if (load) {
+                            if constexpr (l < TileA::LPW)
+                                __builtin_amdgcn_global_load_lds(
+                                    (const __attribute__((address_space(1))) void *)(pa + offA[l]),
+                                    MMBO_LDS_PTR(dst + (wave * TileA::LPW + l) * 1024), 16, 0, 0);
+                            else
+                                __builtin_amdgcn_global_load_lds(
+                                    (const __attribute__((address_space(1))) void *)(pb + offB[l - TileA::LPW]),
+                                    MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024), 16, 0, 0);
+                        }
+                    }
+                });
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
     };
@@ -340,8 +363,8 @@ gemm_ring_kernel(const GemmArgs args)
     // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
     // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free; this
     // wavefront's loads of slices s+2 .. s+DEPTH-1 are in flight.
-    //   iteration s:  issue loads(s+DEPTH) -> buffer s % DEPTH;  MFMAs of slice s from set s&1 interleaved with
-    //                 the reads of slice s+1 -> set (s+1)&1;  wait reads;  wait own loads(s+2);  barrier B_{s+1}.
+    //   iteration s:  MFMAs of slice s from set s&1, interleaved with the loads(s+DEPTH) -> buffer s % DEPTH and the
+    //                 reads of slice s+1 -> set (s+1)&1;  wait reads;  wait own loads(s+2);  barrier B_{s+1}.
     // Loads return in order, so "all but the newest (DEPTH-2) batches" means loads(s+2) have landed; once the
     // tail stops issuing, the wait is for everything.
 #pragma unroll
@@ -358,11 +381,9 @@ gemm_ring_kernel(const GemmArgs args)
     auto step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
         const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
         const bool steady = s + DEPTH < n_slice;
-        if (steady) issue_slice(s + DEPTH, buf);
-        __builtin_amdgcn_sched_barrier(0);
         // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
-        // interleaved block free of branches)
-        mfma_and_read(ca, cb, na, nb, nbuf);
+        // interleaved block free of divergent control flow)
+        mfma_and_read(ca, cb, na, nb, nbuf, steady, s + DEPTH, buf);
         MMBO_WAIT_LGKM0();
         if (steady) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();
