@@ -92,8 +92,8 @@ def cpu_baseline(dtype, m, n, k, hA, hB):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["f16", "f32"], default=None, help="run one leg only (profiling)")
     args = ap.parse_args()
@@ -116,8 +116,9 @@ def main():
     for name, dtype in (("f16", G.F16), ("f32", G.F32)):
         if args.only and args.only != name:
             continue
-        steps = args.steps if name == "f16" else max(3, args.steps // 4)
-        wall_ms, ev_ms, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, args.warmup, seed=1234)
+        steps = args.steps if name == "f16" else max(3, args.steps // 5)
+        warm = args.warmup if name == "f16" else max(2, args.warmup // 5)
+        wall_ms, ev_ms, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, warm, seed=1234)
         rel, limit, host = spot_check(G, dtype, m, n, k, *tensors)
         res[name] = dict(wall_ms=wall_ms, ev_ms=ev_ms, cfg=cfg, rel=rel, limit=limit, steps=steps)
         if name == "f16" and not args.no_cpu:

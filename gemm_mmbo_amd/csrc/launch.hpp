@@ -19,6 +19,9 @@ int staged_lds_bytes();
 template <int DTYPE, int TILE>
 hipError_t launch_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream);
 
+// HGEMM 256 x 256 ring kernel with 64-k units for the k-contiguous operand; NN and TT only, k % 64 == 0, k >= 512.
+hipError_t launch_hgemm_ring_wide(int transA, int transB, const GemmArgs &args, hipStream_t stream);
+
 hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream);
 
 }  // namespace mmbo

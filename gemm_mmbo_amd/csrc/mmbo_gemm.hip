@@ -22,7 +22,8 @@ namespace {
 // slices and A, B are 16-byte aligned; otherwise the call is refused with MMBO_ERR_INVALID_CONFIG.
 constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
 constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
-constexpr int kNumConfigs = kStagedConfigs + kRingConfigs;
+constexpr int kWideConfig = kStagedConfigs + kRingConfigs;      // HGEMM NN/TT 256x256 ring with 64-k units
+constexpr int kNumConfigs = kWideConfig + 1;
 
 struct ConfigRef {
     bool ring;
@@ -31,11 +32,17 @@ struct ConfigRef {
 };
 inline ConfigRef config_ref(int id)
 {
+    if (id == kWideConfig) return {true, 0, 1};                 // same tile and grid as ring tile 0, no split
     if (id < kStagedConfigs) return {false, id % NUM_TILES, kSplits[id / NUM_TILES]};
     id -= kStagedConfigs;
     return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES]};
 }
 inline int ring_config_id(int tile, int split_index) { return kStagedConfigs + tile + NUM_RING_TILES * split_index; }
+
+inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_t k)
+{
+    return dtype == MMBO_F16 && transA == transB && m % 256 == 0 && n % 256 == 0 && k % 64 == 0 && k >= 512;
+}
 
 inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k)
 {
@@ -212,6 +219,12 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
     if (config_id < 0 || config_id >= kNumConfigs) return MMBO_ERR_INVALID_CONFIG;
     std::memset(out, 0, sizeof(*out));
     const ConfigRef c = config_ref(config_id);
+    if (config_id == kWideConfig) {
+        std::snprintf(out->name, sizeof(out->name), "MT256x256x64_WT064x128_W8_GSU01_DTL1_RING4+3U");
+        out->macro_tile_m = 256; out->macro_tile_n = 256; out->depth_u = 64; out->threads = 512;
+        out->wave_tile_m = 64; out->wave_tile_n = 128; out->split_k = 1; out->lds_bytes = 160 * 1024;
+        return MMBO_OK;
+    }
     if (c.ring) {
         const RingRow &r = kRingTiles[c.tile];
         std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d", r.bm, r.bn,
@@ -271,7 +284,10 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
             const RingRow &r = kRingTiles[rt];
             if (r.bm * r.bn > t.bm * t.bn) continue;
             for (int si = 0; si < NUM_SPLITS; ++si)
-                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k)) return ring_config_id(rt, si);
+                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k)) {
+                    if (rt == 0 && si == 0 && wide_ok(dtype, transA, transB, m, n, k)) return kWideConfig;
+                    return ring_config_id(rt, si);
+                }
         }
     }
     return best;
@@ -346,6 +362,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     TileRow r = cref.ring ? TileRow{kRingTiles[cref.tile].bm, kRingTiles[cref.tile].bn, ring_bk(dtype), 0, 0}
                           : tile_row(dtype, cref.tile);
     if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
+    const bool wide = config_id == kWideConfig;
+    if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
     // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
     {
@@ -392,7 +410,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
         if (rc != MMBO_OK) return rc;
     }
     hipError_t e;
-    if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
+    if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
+    else if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
                                          : dispatch_ring<1, 0>(cref.tile, transA, transB, a, s);
     else e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(cref.tile, transA, transB, a, s)
                                : dispatch_tile<1, 0>(cref.tile, transA, transB, a, s);

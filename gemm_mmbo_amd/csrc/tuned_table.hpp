@@ -32,9 +32,9 @@ constexpr TunedRow kTuned[] = {
     {1, 0, 0, 2048, 2048, 2048, 1, 3, 557.1f},
     {0, 0, 1, 44160, 2048, 384, 1, 2, 107.1f},
     {0, 0, 0, 8192, 8192, 8192, 1, 30, 142.0f},
-    {1, 0, 0, 8192, 8192, 8192, 1, 30, 1075.9f},
+    {1, 0, 0, 8192, 8192, 8192, 1, 50, 1190.0f},
     {0, 0, 0, 4096, 4096, 4096, 1, 30, 140.6f},
-    {1, 0, 0, 4096, 4096, 4096, 1, 30, 1018.2f},
+    {1, 0, 0, 4096, 4096, 4096, 1, 50, 1049.0f},
 };
 
 }  // namespace mmbo

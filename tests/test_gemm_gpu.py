@@ -91,12 +91,38 @@ def test_every_config_aligned_interior(dtype):
     import gemm_mmbo_amd as G
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
+        if dtype == F32 and "+3U" in G.config_info(dtype, cid)["name"]:      # an fp16-only kernel
+            with pytest.raises(G.MmboError):
+                U.run_gpu(p, cid)
+            continue
         _run_and_check(p, cid, label=f"config {cid}")
 
 
 def _ring_ids(dtype):
     import gemm_mmbo_amd as G
-    return [c for c in range(G.num_configs(dtype)) if "DTL1" in G.config_info(dtype, c)["name"]]
+    return [c for c in range(G.num_configs(dtype))
+            if "DTL1" in G.config_info(dtype, c)["name"] and "+3U" not in G.config_info(dtype, c)["name"]]
+
+
+def test_wide_unit_ring_kernel_nn_tt():
+    """The HGEMM NN/TT variant that fetches the k-contiguous operand in 64-k units (last config id): K from the
+    shortest it takes (512) up, unit counts that are and are not multiples of the three unit buffers, beta, batches;
+    refused for NT/TN, fp32, short or odd K."""
+    import gemm_mmbo_amd as G
+    cid = G.num_configs(F16) - 1
+    assert "+3U" in G.config_info(F16, cid)["name"]
+    for (ta, tb) in ((0, 0), (1, 1)):
+        for (m, n, k, alpha, beta, batch) in ((256, 256, 512, 1.0, 0.0, 1), (512, 256, 576, 1.5, 0.5, 1), (256, 768, 1024, -1.0, 1.0, 2),
+                                              (768, 512, 4096, 1.0, 0.0, 1), (256, 256, 640, 1.0, 0.0, 1), (256, 512, 704, 1.0, 1.0, 1)):
+            p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=90 + k, dist="normal",
+                          c_fill="uniform" if beta else "nan")
+            _run_and_check(p, cid, label=f"wide {m}x{n}x{k}")
+        assert G.select_config(F16, ta, tb, 8192, 8192, 8192) == cid
+    for (dtype, ta, tb, k) in ((F16, 0, 1, 1024), (F16, 1, 0, 1024), (F32, 0, 0, 1024), (F16, 0, 0, 448), (F16, 0, 0, 1056)):
+        p = U.Problem(dtype, ta, tb, 256, 256, k, 1.0, 0.0, seed=3, c_fill="nan")
+        with pytest.raises(G.MmboError) as e:
+            U.run_gpu(p, cid)
+        assert e.value.status == 5
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
