@@ -1,4 +1,5 @@
-"""Headline benchmark: GEMM TFLOP/s at 8192^3 on one MI355X, fp16 (value) and fp32 (in "also").
+"""Headline benchmark: GEMM TFLOP/s at 8192^3 on one MI355X, fp16 (value) and fp32 (in "also"); "also" further
+carries the reference's own workload, DGEMM NT 44160 x 2048 x 384 with alpha = -1, beta = 1, and DGEMM at 8192^3.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
@@ -16,7 +17,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 METRIC = "GEMM TFLOP/s + % of MFMA peak, fp16 & fp32 at 8192^3, 1 MI355X"
-PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3}      # MI355X published dense matrix peaks
+PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}      # MI355X published dense matrix peaks
 # Bytes per launch that crossed the L2 <-> fabric boundary, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
 # this same command (each scaled by the counter's reading for a plain elementwise pass of known size; the
 # summaries with the commands are profiles/hgemm_ring_wide_8192.txt and profiles/sgemm_ring_8192.txt).
@@ -74,6 +75,60 @@ def spot_check(G, dtype, m, n, k, A, B, C):
     return rel, U.tol(dtype, k), (hA, hB)
 
 
+def dgemm_legs(G, torch, steps, warmup):
+    """fp64: the reference's HPL trailing update (src/gemm/test.cc:20-21, src/gemm/run.sh:2-5: NT, alpha = -1,
+    beta = 1, inputs in [0, 1)) and NN 8192^3.  Returns the entries for "also"."""
+    import numpy as np
+    from oracle import oracle as O
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import util as U
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4321)
+    out = {}
+    for tag, (ta, tb, m, n, k, alpha, beta) in (("hpl", (0, 1, 44160, 2048, 384, -1.0, 1.0)),
+                                                ("8192", (0, 0, 8192, 8192, 8192, 1.0, 0.0))):
+        lda, ldb = (k if ta else m), (n if tb else k)
+        A = torch.rand(m * k, device="cuda", generator=gen, dtype=torch.float64)
+        B = torch.rand(k * n, device="cuda", generator=gen, dtype=torch.float64)
+        C0 = torch.rand(m * n, device="cuda", generator=gen, dtype=torch.float64)
+        C = C0.clone()
+        cid = G.select_config(G.F64, ta, tb, m, n, k, 1)
+        nsteps = max(3, steps // 5) if tag == "8192" else steps
+        for _ in range(max(2, warmup // 4)):
+            G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(nsteps):
+            G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / nsteps
+        # parity on a band of 64 rows of one fresh application (beta = 1 accumulates over the timed launches)
+        C.copy_(C0)
+        G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
+        torch.cuda.synchronize()
+        r0 = 4000
+        hA, hB, hC0, hC = A.cpu().numpy(), B.cpu().numpy(), C0.cpu().numpy(), C.cpu().numpy()
+        want = O.gemm_f64(O.F64, ta, tb, 64, n, k, alpha, hA[r0:], lda, hB, ldb, beta, hC0[r0:] if beta else None, m)
+        rel, _ = O.max_rel_err(O.F64, hC[r0:], m, want, 64, n, floor=float(np.sqrt(np.mean(want * want))))
+        tf = 2.0 * m * n * k / ms * 1e-9
+        out[f"fp64_{tag}_tflops"] = round(tf, 2)
+        out[f"fp64_{tag}_ms_per_step"] = round(ms, 4)
+        out[f"fp64_{tag}_frac_of_peak"] = round(tf / PEAK_TFLOPS["f64"], 4)
+        out[f"fp64_{tag}_tile_config"] = G.config_info(G.F64, cid)["name"]
+        out[f"fp64_{tag}_max_rel_err"] = float(f"{rel:.3e}")
+        out[f"fp64_{tag}_rel_err_limit"] = float(f"{U.tol(U.F64, k):.3e}")
+        if tag == "hpl":
+            out["fp64_hpl_workload"] = "DGEMM NT M=44160 N=2048 K=384 alpha=-1 beta=1, A,B,C ~ U[0,1)"
+            out["fp64_hpl_algorithmic_GBps"] = round((m * k + k * n + 2 * m * n) * 8 / ms * 1e-6, 1)
+        del A, B, C, C0
+        torch.cuda.empty_cache()
+    out["fp64_peak"] = PEAK_TFLOPS["f64"]
+    return out
+
+
 def cpu_baseline(dtype, m, n, k, hA, hB):
     """The oracle's native-precision CPU GEMM (fp16 operands widened to fp32, fp32 multiply-add chains) on
     the same operands, all host cores, whole problem once."""
@@ -95,7 +150,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["f16", "f32"], default=None, help="run one leg only (profiling)")
+    ap.add_argument("--only", choices=["f16", "f32", "f64"], default=None, help="run one leg only (profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this library runs one GEMM on one GPU; --gpus must be 1 "
@@ -126,9 +181,13 @@ def main():
         del tensors, host
         torch.cuda.empty_cache()
 
+    f64 = dgemm_legs(G, torch, args.steps, args.warmup) if args.only in (None, "f64") else {}
+    if args.only == "f64":
+        print(json.dumps({"metric": METRIC, "also": f64}))
+        return
     ceilings = {}
     if not args.only:
-        for name, dtype in (("f16", G.F16), ("f32", G.F32)):
+        for name, dtype in (("f16", G.F16), ("f32", G.F32), ("f64", G.F64)):
             for rnd in (0, 1):
                 tf, mhz = G.probe_mfma_ceiling(dtype, bool(rnd))
                 ceilings[f"{name}_{'random' if rnd else 'ones'}_operands"] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
@@ -165,6 +224,10 @@ def main():
                        "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
                        "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
                        "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}
+    if f64:
+        out.setdefault("also", {}).update(f64)
+        out["parity_ok"] = bool(out["parity_ok"] and f64["fp64_hpl_max_rel_err"] <= f64["fp64_hpl_rel_err_limit"]
+                                and f64["fp64_8192_max_rel_err"] <= f64["fp64_8192_rel_err_limit"])
     print(json.dumps(out))
     if not out["parity_ok"]:
         sys.exit(3)

@@ -10,7 +10,7 @@ There is no CPU path: if the HIP library has not been built this module raises o
 import ctypes
 import os
 
-F32, F16 = 0, 1
+F32, F16, F64 = 0, 1, 2
 OP_N, OP_T = 0, 1
 CONFIG_AUTO = -1
 
@@ -102,16 +102,22 @@ def _stream_handle(stream):
     return ctypes.c_void_p(stream.cuda_stream)
 
 
+def _scalars(dtype, alpha, beta):
+    """alpha and beta in the type the C ABI reads them in: double for F64, float otherwise."""
+    t = ctypes.c_double if dtype == F64 else ctypes.c_float
+    return t(alpha), t(beta)
+
+
 def gemm(dtype, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, config_id=CONFIG_AUTO, stream=None):
     """C = alpha*op(A)*op(B) + beta*C on the current device; asynchronous on `stream`."""
-    al, be = ctypes.c_float(alpha), ctypes.c_float(beta)
+    al, be = _scalars(dtype, alpha, beta)
     _check(lib().mmbo_gemm(dtype, transA, transB, m, n, k, ctypes.byref(al), _devptr(A), lda, _devptr(B), ldb,
                            ctypes.byref(be), _devptr(C), ldc, config_id, _stream_handle(stream)))
 
 
 def gemm_strided_batched(dtype, transA, transB, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc,
                          strideC, batch, config_id=CONFIG_AUTO, stream=None):
-    al, be = ctypes.c_float(alpha), ctypes.c_float(beta)
+    al, be = _scalars(dtype, alpha, beta)
     _check(lib().mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k, ctypes.byref(al), _devptr(A), lda,
                                            strideA, _devptr(B), ldb, strideB, ctypes.byref(be), _devptr(C), ldc,
                                            strideC, batch, config_id, _stream_handle(stream)))
@@ -165,6 +171,11 @@ def naive_sgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId=CONFIG_AU
     gemm(F32, OP_N, OP_N, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId)
 
 
+def naive_dgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId=CONFIG_AUTO):
+    """The reference's own entry point (src/gemm/gemm.h:4-5): DGEMM, A not transposed, B transposed."""
+    gemm(F64, OP_N, OP_T, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId)
+
+
 def naive_hgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId=CONFIG_AUTO):
     gemm(F16, OP_N, OP_N, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId)
 
@@ -177,3 +188,4 @@ def _front_end(dtype, ta, tb):
 
 sgemm_NN, sgemm_NT, sgemm_TN, sgemm_TT = (_front_end(F32, a, b) for a in (0, 1) for b in (0, 1))
 hgemm_NN, hgemm_NT, hgemm_TN, hgemm_TT = (_front_end(F16, a, b) for a in (0, 1) for b in (0, 1))
+dgemm_NN, dgemm_NT, dgemm_TN, dgemm_TT = (_front_end(F64, a, b) for a in (0, 1) for b in (0, 1))

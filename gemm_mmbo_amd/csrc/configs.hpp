@@ -34,6 +34,17 @@ constexpr TileRow kTilesF16[NUM_TILES] = {
     { 32,  32, 64, 1, 1},
 };
 
+// fp64 (dgemm.hpp): 16x16 MFMA blocks, no split-K; config id = row.
+constexpr int NUM_F64_TILES = 6;
+constexpr TileRow kTilesF64[NUM_F64_TILES] = {
+    {128, 128, 16, 2, 2},
+    {256, 128, 16, 4, 2},
+    { 64,  64, 16, 2, 2},
+    { 32,  32, 16, 2, 2},
+    {128, 128, 16, 4, 2},     // 64 accumulator registers per lane: four wavefronts per SIMD overlap C traffic with MFMAs
+    {128,  64, 16, 2, 2},
+};
+
 constexpr const TileRow &tile_row(int dtype, int tile) { return dtype == 0 ? kTilesF32[tile] : kTilesF16[tile]; }
 
 // Ring kernel tiles (gemm_ring.hpp), the same for both element types; depthU is 32 (fp16) / 16 (fp32).

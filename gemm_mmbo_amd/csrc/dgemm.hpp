@@ -1,0 +1,201 @@
+// DGEMM for gfx950 on v_mfma_f64_16x16x4_f64: the reference's own element type and workload
+// (src/gemm/gemm.h:4-5,47-48 naive_dgemm / dgemm_NT; the HPL trailing update of src/gemm/run.sh:2-5).
+//
+// Same structure as the staged fp32/fp16 kernel (global loads into registers one stage ahead, padded
+// double-buffered LDS tile, one barrier per stage; edges, K tail and unaligned operands through the predicated
+// loader), with 16 x 16 MFMA blocks: an fp64 MFMA takes 64 clocks for 2,048 flops, so one 64-bit LDS read per
+// operand per MFMA and a single-stage prefetch keep the pipes fed.
+//
+// Register layout of v_mfma_f64_16x16x4_f64 (checked on the device): operand lane l supplies row (column)
+// l%16 at k = l/16; result element e of lane l is D[4*e + l/16][l%16].  A lane's four results are therefore
+// four rows 4 apart.  The A fragment is read with its 16 rows permuted, MFMA row r <- tile row 4*(r%4) + r/4,
+// which turns them into the four CONSECUTIVE rows 4*(l/16) .. +3 of column l%16: 32 contiguous bytes per lane,
+// a full 128-byte line per column across the four lane groups.
+#pragma once
+
+#include "gemm_staged.hpp"
+
+namespace mmbo {
+
+template <bool KC, int LDS_LD>
+__device__ inline uint32_t dfrag_lane_off(int lane, int row0, bool permute_rows)
+{
+    int r = lane & 15, g = lane >> 4;
+    if (permute_rows) r = 4 * (r & 3) + (r >> 2);
+    if (KC) return (uint32_t)((row0 + r) * LDS_LD + g) * 8;
+    return (uint32_t)(g * LDS_LD + row0 + r) * 8;
+}
+
+// fragment of 16-row block rblk for k = 4*kk + lane/16
+template <bool KC, int LDS_LD>
+__device__ inline double dread_frag(const char *lds, uint32_t lane_off, int rblk, int kk)
+{
+    uint32_t off = lane_off + (uint32_t)(KC ? rblk * 16 * LDS_LD + kk * 4 : kk * 4 * LDS_LD + rblk * 16) * 8;
+    return *reinterpret_cast<const double *>(lds + off);
+}
+
+template <bool TA, bool TB, int BM, int BN, int BK, int WM, int WN>
+struct DgemmCfg {
+    static constexpr int NT = WM * WN * 64;
+    static constexpr int TM = BM / WM, TN = BN / WN;
+    static constexpr int FM = TM / 16, FN = TN / 16;
+    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA block");
+    static_assert(BK % 4 == 0, "depthU must be a multiple of the MFMA's k");
+    using TileA = OperandTile<double, TA, BM, BK, NT>;
+    using TileB = OperandTile<double, !TB, BN, BK, NT>;
+    static constexpr int STAGE_BYTES = TileA::LDS_BYTES + TileB::LDS_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+};
+
+// C = alpha*acc + beta*C for one wavefront's FM x FN blocks; acc[i][j][e] is
+// C(wrow0 + 16*i + 4*(lane/16) + e, wcol0 + 16*j + lane%16).  beta == 0 never reads C
+// (src/gemm/ref/Kernels.cpp:87); alpha*acc first, then fma(beta, C, .), as the reference's epilogue.
+template <int FM, int FN>
+__device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmArgs &args, uint32_t wrow0,
+                                        uint32_t wcol0, uint32_t batch, int lane)
+{
+    const uint32_t m = args.m, n = args.n, ldc = args.ldc;
+    const double alpha = args.alpha_d, beta = args.beta_d;
+    const int g = lane >> 4, cl = lane & 15;
+    double *C = static_cast<double *>(args.C) + (int64_t)batch * args.strideC;
+    const bool vec_c = args.vec_c != 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            uint32_t col = wcol0 + j * 16 + cl;
+            uint32_t row = wrow0 + i * 16 + 4 * g;
+            if (col >= n || row >= m) continue;
+            double *p = C + (size_t)col * ldc + row;
+            double v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][e];
+            if (vec_c && row + 4 <= m) {
+                if (beta != 0.0) {
+                    f64x2 c0 = *reinterpret_cast<const f64x2 *>(p), c1 = *reinterpret_cast<const f64x2 *>(p + 2);
+                    v[0] = __builtin_fma(beta, c0[0], v[0]);
+                    v[1] = __builtin_fma(beta, c0[1], v[1]);
+                    v[2] = __builtin_fma(beta, c1[0], v[2]);
+                    v[3] = __builtin_fma(beta, c1[1], v[3]);
+                }
+                *reinterpret_cast<f64x2 *>(p) = f64x2{v[0], v[1]};
+                *reinterpret_cast<f64x2 *>(p + 2) = f64x2{v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (row + e < m) {
+                        double o = v[e];
+                        if (beta != 0.0) o = __builtin_fma(beta, p[e], o);
+                        p[e] = o;
+                    }
+            }
+        }
+}
+
+template <bool TA, bool TB, int BM, int BN, int BK, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64, 2)      // two wavefronts per SIMD: at most 256 registers per lane
+dgemm_kernel(const GemmArgs args)
+{
+    using Cfg = DgemmCfg<TA, TB, BM, BN, BK, WM, WN>;
+    using TileA = typename Cfg::TileA;
+    using TileB = typename Cfg::TileB;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN, ESZ = 8, NKK = BK / 4;
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+
+    uint32_t wg0, wg1;
+    wg_remap(blockIdx.x, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
+    const uint32_t batch = blockIdx.z;
+
+    const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
+    const int rows_a = (int)min((uint32_t)BM, args.m - row0);
+    const int rows_b = (int)min((uint32_t)BN, args.n - col0);
+    const uint32_t k_len = args.k;
+    const int n_full = (int)(k_len / BK);
+    const int k_tail = (int)(k_len % BK);
+    const int n_iter = n_full + (k_tail ? 1 : 0);
+
+    const uint32_t lda = args.lda, ldb = args.ldb;
+    const char *gA = static_cast<const char *>(args.A) +
+                     ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda : (int64_t)row0)) * ESZ;
+    const char *gB = static_cast<const char *>(args.B) +
+                     ((int64_t)batch * args.strideB + (TB ? (int64_t)col0 : (int64_t)col0 * ldb)) * ESZ;
+    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * ESZ;
+    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * ESZ;
+
+    uint32_t offA[TileA::NCH], offB[TileB::NCH];
+#pragma unroll
+    for (int c = 0; c < TileA::NCH; ++c) offA[c] = TileA::goff(tid, c, lda);
+#pragma unroll
+    for (int c = 0; c < TileB::NCH; ++c) offB[c] = TileB::goff(tid, c, ldb);
+
+    const bool fast = rows_a == BM && rows_b == BN && args.vec_a && args.vec_b;
+
+    u32x4 ra[TileA::NCH], rb[TileB::NCH];
+    auto load_stage = [&](int it) {
+        const char *pa = gA + (int64_t)it * stepA;
+        const char *pb = gB + (int64_t)it * stepB;
+        if (fast && it < n_full) {
+            TileA::load_fast(ra, pa, offA);
+            TileB::load_fast(rb, pb, offB);
+        } else {
+            int kvalid = it < n_full ? BK : k_tail;
+            TileA::load_slow(ra, pa, offA, tid, lda, rows_a, kvalid, args.vec_a != 0);
+            TileB::load_slow(rb, pb, offB, tid, ldb, rows_b, kvalid, args.vec_b != 0);
+        }
+    };
+
+    f64x4 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0};
+
+    const uint32_t fa_off = dfrag_lane_off<TA, TileA::LDS_LD>(lane, wm * Cfg::TM, true);
+    const uint32_t fb_off = dfrag_lane_off<!TB, TileB::LDS_LD>(lane, wn * Cfg::TN, false) + TileA::LDS_BYTES;
+
+    if (n_iter > 0) {
+        load_stage(0);
+        TileA::store_lds(ra, lds, tid);
+        TileB::store_lds(rb, lds + TileA::LDS_BYTES, tid);
+    }
+    __syncthreads();
+
+    int cur = 0;
+    for (int it = 0; it < n_iter; ++it) {
+        const bool more = it + 1 < n_iter;
+        if (more) load_stage(it + 1);
+
+        const char *st = lds + cur * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+            double fa[FM], fb[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) fa[i] = dread_frag<TA, TileA::LDS_LD>(st, fa_off, i, kk);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) fb[j] = dread_frag<!TB, TileB::LDS_LD>(st, fb_off, j, kk);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (more) {
+            char *nx = lds + (cur ^ 1) * Cfg::STAGE_BYTES;
+            TileA::store_lds(ra, nx, tid);
+            TileB::store_lds(rb, nx + TileA::LDS_BYTES, tid);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    dgemm_write_back<FM, FN>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, lane);
+}
+
+}  // namespace mmbo

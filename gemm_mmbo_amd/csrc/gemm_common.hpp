@@ -17,6 +17,8 @@ typedef _Float16 f16x4  __attribute__((ext_vector_type(4)));
 typedef short    i16x4  __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4  __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2  __attribute__((ext_vector_type(2)));
+typedef double   f64x4  __attribute__((ext_vector_type(4)));
+typedef double   f64x2  __attribute__((ext_vector_type(2)));
 
 #define MMBO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
@@ -30,6 +32,7 @@ struct GemmArgs {
     float *ws;              // split-K partial sums: [split][batch][n][m] fp32, dense
     float alpha;
     float beta;
+    double alpha_d, beta_d; // the fp64 kernels' scalars (the reference's own type, src/gemm/gemm.h:31-32)
     uint32_t m, n, k;       // sizeI, sizeJ, sizeL
     uint32_t lda, ldb, ldc; // strideA1L/strideB1L/strideC1J, in elements
     int64_t strideA, strideB, strideC;   // batch strides in elements (strideA2K/B2K/C2K)
@@ -76,6 +79,12 @@ template <> struct ElemTraits<float> {
     static constexpr int KG = 8;       // k extent covered by one round of LDS fragment reads
     static constexpr int PAD_KC = 4;   // row padding (elements) of a k-contiguous LDS tile: 16 B
     static constexpr int PAD_RC = 8;   // row padding of a row-contiguous LDS tile
+};
+template <> struct ElemTraits<double> {
+    static constexpr int VEC = 2;
+    static constexpr int KG = 4;       // one v_mfma_f64_16x16x4 consumes four k values
+    static constexpr int PAD_KC = 2;   // 16 B: 16 rows x 2 k of one 64-bit fragment read land on 64 distinct banks
+    static constexpr int PAD_RC = 16;  // row length = 16 mod 32 doubles: two k-rows of a read sit 32 banks apart
 };
 template <> struct ElemTraits<half_t> {
     static constexpr int VEC = 8;

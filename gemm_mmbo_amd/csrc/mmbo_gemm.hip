@@ -37,6 +37,7 @@ inline ConfigRef config_ref(int id)
     id -= kStagedConfigs;
     return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES]};
 }
+inline bool valid_dtype(int dtype) { return dtype == MMBO_F32 || dtype == MMBO_F16 || dtype == MMBO_F64; }
 inline int ring_config_id(int tile, int split_index) { return kStagedConfigs + tile + NUM_RING_TILES * split_index; }
 
 inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_t k)
@@ -115,6 +116,22 @@ hipError_t dispatch_ring(int tile, int ta, int tb, const GemmArgs &a, hipStream_
     return hipErrorInvalidValue;
 }
 
+template <int TILE>
+hipError_t dispatch_dgemm(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
+{
+    if (tile == TILE) return launch_dgemm<TILE>(ta, tb, a, s);
+    if constexpr (TILE + 1 < NUM_F64_TILES) return dispatch_dgemm<TILE + 1>(tile, ta, tb, a, s);
+    return hipErrorInvalidValue;
+}
+
+template <int TILE>
+int dgemm_lds_bytes_of(int tile)
+{
+    if (tile == TILE) return dgemm_lds_bytes<TILE>();
+    if constexpr (TILE + 1 < NUM_F64_TILES) return dgemm_lds_bytes_of<TILE + 1>(tile);
+    return 0;
+}
+
 template <int DTYPE, int TILE>
 int lds_bytes_of(int tile)
 {
@@ -169,6 +186,32 @@ double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, 
     return t;
 }
 
+// fp64: same model, one stage of prefetch, 64 MACs per clock per CU, no split-K.
+double model_time_f64(int tile, size_t m, size_t n, size_t k, int batch)
+{
+    const TileRow &r = kTilesF64[tile];
+    const double cus = 256.0, mac_per_clk_cu = 64.0, hbm_bytes_per_clk = 3300.0, load_latency = 1700.0;
+    double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch;
+    int lds = dgemm_lds_bytes_of<0>(tile);
+    int per_cu = 160 * 1024 / (lds > 0 ? lds : 1);
+    int thr = r.wm * r.wn * 64;
+    if (per_cu > 1024 / thr) per_cu = 1024 / thr;      // the large tiles need more than 128 registers per lane
+    if (per_cu < 1) per_cu = 1;
+    double slots = cus * per_cu;
+    double rounds = (double)ceil_div((size_t)tiles, (size_t)slots);
+    double resident = tiles >= slots ? per_cu : (tiles > cus ? tiles / cus : 1.0);
+    double wave_cost = r.bm * r.bn / (r.wm * r.wn) >= 64 * 64 ? 1.0 : (r.bm >= 64 ? 1.1 : 1.5);
+    double stage_mfma = (double)r.bm * r.bn * r.bk * wave_cost / mac_per_clk_cu;
+    double stage = stage_mfma * resident > load_latency ? stage_mfma * resident : load_latency;
+    double stages = (double)ceil_div(k ? k : 1, (size_t)r.bk);
+    double epilogue = (double)r.bm * r.bn * 8.0 * resident / 24.0;
+    if (per_cu * thr >= 1024) epilogue *= 0.6;          // four wavefronts per SIMD hide part of the C traffic
+    double compute = rounds * (stages * stage + load_latency + epilogue);
+    double bytes = ((double)m * k + (double)k * n + (double)m * n) * batch * 8.0;
+    double t = compute > bytes / hbm_bytes_per_clk ? compute : bytes / hbm_bytes_per_clk;
+    return t + 9000.0;
+}
+
 }  // namespace
 
 hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream)
@@ -208,16 +251,25 @@ const char *mmbo_status_string(int status)
 
 int mmbo_num_configs(int dtype)
 {
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
-    return kNumConfigs;
+    if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
+    return dtype == MMBO_F64 ? NUM_F64_TILES : kNumConfigs;
 }
 
 int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
 {
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if (!valid_dtype(dtype)) return MMBO_ERR_INVALID_DTYPE;
     if (!out) return MMBO_ERR_NULL_POINTER;
-    if (config_id < 0 || config_id >= kNumConfigs) return MMBO_ERR_INVALID_CONFIG;
+    if (config_id < 0 || config_id >= mmbo_num_configs(dtype)) return MMBO_ERR_INVALID_CONFIG;
     std::memset(out, 0, sizeof(*out));
+    if (dtype == MMBO_F64) {
+        const TileRow &r = kTilesF64[config_id];
+        std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU01_MFMA16x16x4", r.bm, r.bn,
+                      r.bk, r.bm / r.wm, r.bn / r.wn, r.wm * r.wn);
+        out->macro_tile_m = r.bm; out->macro_tile_n = r.bn; out->depth_u = r.bk; out->threads = r.wm * r.wn * 64;
+        out->wave_tile_m = r.bm / r.wm; out->wave_tile_n = r.bn / r.wn; out->split_k = 1;
+        out->lds_bytes = dgemm_lds_bytes_of<0>(config_id);
+        return MMBO_OK;
+    }
     const ConfigRef c = config_ref(config_id);
     if (config_id == kWideConfig) {
         std::snprintf(out->name, sizeof(out->name), "MT256x256x64_WT064x128_W8_GSU01_DTL1_RING4+3U");
@@ -256,10 +308,23 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
 
 int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch)
 {
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return -MMBO_ERR_INVALID_DTYPE;
+    if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
     if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
     if (batch < 0) return -MMBO_ERR_INVALID_SIZE;
     if (m == 0 || n == 0 || batch == 0) return 0;
+    if (dtype == MMBO_F64) {
+        for (const TunedRow &t : kTuned)
+            if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
+                t.batch == batch)
+                return t.config_id;
+        int best = 0;
+        double best_t = 0.0;
+        for (int tile = 0; tile < NUM_F64_TILES; ++tile) {
+            double t = model_time_f64(tile, m, n, k, batch);
+            if (best_t == 0.0 || t < best_t) { best_t = t; best = tile; }
+        }
+        return best;
+    }
     for (const TunedRow &t : kTuned)
         if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
             t.batch == batch)
@@ -329,7 +394,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
                               const void *B, size_t ldb, long long strideB, const void *beta, void *C,
                               size_t ldc, long long strideC, int batch, int config_id, void *stream)
 {
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if (!valid_dtype(dtype)) return MMBO_ERR_INVALID_DTYPE;
     if ((transA & ~1) || (transB & ~1)) return MMBO_ERR_INVALID_OP;
     if (!alpha || !beta) return MMBO_ERR_NULL_POINTER;
     const size_t kMaxDim = 0x7FFFFFFFull;
@@ -343,26 +408,28 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
             return MMBO_ERR_INVALID_SIZE;
     }
     if (strideA < 0 || strideB < 0 || strideC < 0) return MMBO_ERR_INVALID_SIZE;
-    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= kNumConfigs))
+    if (config_id != MMBO_CONFIG_AUTO && (config_id < 0 || config_id >= mmbo_num_configs(dtype)))
         return MMBO_ERR_INVALID_CONFIG;
     if (m == 0 || n == 0 || batch == 0) return MMBO_OK;          // nothing to write
     if (!C) return MMBO_ERR_NULL_POINTER;
     if (k != 0 && (!A || !B)) return MMBO_ERR_NULL_POINTER;
 
-    const float alpha_f = *static_cast<const float *>(alpha);
-    const float beta_f = *static_cast<const float *>(beta);
+    const bool f64 = dtype == MMBO_F64;
+    const double alpha_d = f64 ? *static_cast<const double *>(alpha) : (double)*static_cast<const float *>(alpha);
+    const double beta_d = f64 ? *static_cast<const double *>(beta) : (double)*static_cast<const float *>(beta);
+    const float alpha_f = (float)alpha_d, beta_f = (float)beta_d;
 
     if (config_id == MMBO_CONFIG_AUTO) {
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
     }
-    const ConfigRef cref = config_ref(config_id);
-    const size_t esz = dtype == MMBO_F32 ? 4 : 2;
+    const ConfigRef cref = f64 ? ConfigRef{false, config_id, 1} : config_ref(config_id);
+    const size_t esz = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
     int split = cref.split;
-    TileRow r = cref.ring ? TileRow{kRingTiles[cref.tile].bm, kRingTiles[cref.tile].bn, ring_bk(dtype), 0, 0}
+    TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{kRingTiles[cref.tile].bm, kRingTiles[cref.tile].bn, ring_bk(dtype), 0, 0}
                           : tile_row(dtype, cref.tile);
     if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
-    const bool wide = config_id == kWideConfig;
+    const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
     // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
@@ -386,6 +453,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     std::memset(&a, 0, sizeof(a));
     a.A = A; a.B = B; a.C = C; a.ws = nullptr;
     a.alpha = alpha_f; a.beta = beta_f;
+    a.alpha_d = alpha_d; a.beta_d = beta_d;
     a.m = (uint32_t)m; a.n = (uint32_t)n; a.k = (uint32_t)k;
     a.lda = (uint32_t)lda; a.ldb = (uint32_t)ldb; a.ldc = (uint32_t)ldc;
     a.strideA = strideA; a.strideB = strideB; a.strideC = strideC;
@@ -410,7 +478,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
         if (rc != MMBO_OK) return rc;
     }
     hipError_t e;
-    if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
+    if (f64) e = dispatch_dgemm<0>(cref.tile, transA, transB, a, s);
+    else if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
     else if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
                                          : dispatch_ring<1, 0>(cref.tile, transA, transB, a, s);
     else e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(cref.tile, transA, transB, a, s)

@@ -17,6 +17,39 @@ namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(512) mfma_ceiling_kernel_f64(const uint32_t *src, float *out, long long *clk, int iters)
+{
+    f64x4 acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = f64x4{0.0, 0.0, 0.0, 0.0};
+    union { uint32_t u[2]; double d; } a[4], b[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            a[q].u[e] = src[(threadIdx.x * 4 + q) * 2 + e];
+            b[q].u[e] = src[8192 + (threadIdx.x * 4 + q) * 2 + e];
+        }
+    const long long t0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i % 4].d, b[(i / 2) % 4].d, acc[i], 0, 0, 0);
+    }
+    const long long t1 = clock64(), w1 = wall_clock64();
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s += acc[i][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = (float)s;
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        clk[0] = t1 - t0;
+        clk[1] = w1 - w0;
+    }
+}
 
 template <bool F16>
 __global__ void __launch_bounds__(512) mfma_ceiling_kernel(const uint32_t *src, float *out, long long *clk, int iters)
@@ -67,13 +100,13 @@ uint64_t mix64(uint64_t z)
 
 extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *tflops, double *shader_mhz)
 {
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return MMBO_ERR_INVALID_DTYPE;
+    if (dtype != MMBO_F32 && dtype != MMBO_F16 && dtype != MMBO_F64) return MMBO_ERR_INVALID_DTYPE;
     if (!tflops || !shader_mhz) return MMBO_ERR_NULL_POINTER;
     hipDeviceProp_t prop;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MMBO_ERR_NO_DEVICE;
     const int blocks = prop.multiProcessorCount, threads = 512;
-    const int iters = dtype == MMBO_F16 ? 20000 : 10000;
+    const int iters = dtype == MMBO_F16 ? 20000 : dtype == MMBO_F32 ? 10000 : 5000;
 
     // operands: 1.0 everywhere, or uniform [-0.3, 0.3) with every mantissa bit in play
     std::vector<uint32_t> h(16384);
@@ -89,6 +122,15 @@ extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *t
             __builtin_memcpy(&lb, &lo, 2);
             __builtin_memcpy(&hb, &hi, 2);
             h[i] = (uint32_t)lb | ((uint32_t)hb << 16);
+        } else if (dtype == MMBO_F64) {
+            if (i % 2) continue;                   // a double takes words i, i + 1
+            double v = 1.0;
+            if (random_operands) {
+                uint64_t r = mix64(i);
+                uint64_t bits = 0x3FD0000000000000ull | (r & 0x000FFFFFFFFFFFFFull) | ((r >> 63) << 63);   // +-[0.25, 0.5)
+                __builtin_memcpy(&v, &bits, 8);
+            }
+            __builtin_memcpy(&h[i], &v, 8);
         } else {
             float v = 1.0f;
             if (random_operands) v = (float)(((double)(mix64(i) >> 11) / 9007199254740992.0 * 2.0 - 1.0) * 0.3);
@@ -109,7 +151,8 @@ extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *t
         float ms = 0.0f;
         for (int rep = 0; rep < 3; ++rep) {      // the clock settles over the first launches; the last one counts
             (void)hipEventRecord(e0, nullptr);
-            if (dtype == MMBO_F16) hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
+            if (dtype == MMBO_F64) hipLaunchKernelGGL(mfma_ceiling_kernel_f64, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
+            else if (dtype == MMBO_F16) hipLaunchKernelGGL(mfma_ceiling_kernel<true>, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
             else hipLaunchKernelGGL(mfma_ceiling_kernel<false>, dim3(blocks), dim3(threads), 0, nullptr, d_src, d_out, d_clk, iters);
             (void)hipEventRecord(e1, nullptr);
             if (hipEventSynchronize(e1) != hipSuccess) break;
@@ -117,7 +160,7 @@ extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *t
         }
         long long c[2] = {0, 1};
         if (hipMemcpy(c, d_clk, 16, hipMemcpyDeviceToHost) != hipSuccess || ms <= 0.0f) break;
-        const double flops_per_mfma = dtype == MMBO_F16 ? 32768.0 : 4096.0;
+        const double flops_per_mfma = dtype == MMBO_F16 ? 32768.0 : dtype == MMBO_F32 ? 4096.0 : 2048.0;
         *tflops = (double)blocks * (threads / 64) * iters * 8.0 * flops_per_mfma / (ms * 1e-3) * 1e-12;
         *shader_mhz = c[1] > 0 ? (double)c[0] / (double)c[1] * 100.0 : 0.0;
         rc = MMBO_OK;

@@ -7,8 +7,9 @@
 //           the 23 Tensile kernels)
 //   type 2: in the reference this timed rocBLAS; this library has no third-party GEMM to compare with
 //           and says so
-//   transA/transB: N or T (default N T, the reference's only layout); dtype: s (fp32) or h (fp16);
-//   alpha, beta default to the reference's -1 and 1 (src/gemm/benchmark.cc:20).
+//   transA/transB: N or T (default N T, the reference's only layout); dtype: s (fp32), h (fp16) or
+//   d (fp64, the reference's element type); alpha, beta default to the reference's -1 and 1
+//   (src/gemm/benchmark.cc:20).
 //
 // TFLOP/s = 1e-12 * 2*M*N*K*batch / t (src/gemm/benchmark.cc:98), t from a blocking-sync event pair on the
 // null stream (src/gemm/common.h:4-18) around `reps` launches after one warm-up.  The reference timed one
@@ -20,7 +21,7 @@
 #include "common.h"
 #include "gemm.h"
 
-static double peak_tflops(int dtype) { return dtype == MMBO_F16 ? 2500.0 : 157.3; }
+static double peak_tflops(int dtype) { return dtype == MMBO_F16 ? 2500.0 : dtype == MMBO_F64 ? 78.6 : 157.3; }
 
 int main(int argc, char **argv)
 {
@@ -35,23 +36,30 @@ int main(int argc, char **argv)
                  ldc = std::strtoull(argv[7], NULL, 10);
     const int ta = argc > 8 && (argv[8][0] == 'T' || argv[8][0] == 't') ? MMBO_OP_T : MMBO_OP_N;
     const int tb = argc > 9 ? ((argv[9][0] == 'T' || argv[9][0] == 't') ? MMBO_OP_T : MMBO_OP_N) : MMBO_OP_T;
-    const int dtype = argc > 10 && (argv[10][0] == 'h' || argv[10][0] == 'H') ? MMBO_F16 : MMBO_F32;
+    const char dch = argc > 10 ? argv[10][0] : 's';
+    const int dtype = (dch == 'h' || dch == 'H') ? MMBO_F16 : (dch == 'd' || dch == 'D') ? MMBO_F64 : MMBO_F32;
     const int batch = argc > 11 ? std::atoi(argv[11]) : 1;
-    float alpha = argc > 12 ? (float)std::atof(argv[12]) : -1.0f;
-    float beta = argc > 13 ? (float)std::atof(argv[13]) : 1.0f;
+    const double alpha_d = argc > 12 ? std::atof(argv[12]) : -1.0, beta_d = argc > 13 ? std::atof(argv[13]) : 1.0;
+    const float alpha_f = (float)alpha_d, beta_f = (float)beta_d;
+    // the C ABI reads the scalars in double for fp64 and in float otherwise
+    const void *alpha = dtype == MMBO_F64 ? (const void *)&alpha_d : (const void *)&alpha_f;
+    const void *beta = dtype == MMBO_F64 ? (const void *)&beta_d : (const void *)&beta_f;
     if (type == 2) {
         std::printf("type 2 (third-party BLAS comparison) is not part of this library\n");
         return 0;
     }
 
-    const size_t esz = dtype == MMBO_F16 ? 2 : 4;
+    const size_t esz = dtype == MMBO_F16 ? 2 : dtype == MMBO_F64 ? 8 : 4;
     const size_t a_elems = lda * (ta ? M : K), b_elems = ldb * (tb ? K : N), c_elems = ldc * N;
     // host fill like the reference's (src/gemm/benchmark.cc:45-53: rand() in [0,1], A then B then C)
     std::vector<unsigned char> hA(a_elems * batch * esz), hB(b_elems * batch * esz), hC(c_elems * batch * esz);
     auto fill = [&](std::vector<unsigned char> &buf, size_t count) {
         for (size_t i = 0; i < count; ++i) {
             float v = (float)std::rand() / (float)RAND_MAX;
-            if (dtype == MMBO_F16) {
+            if (dtype == MMBO_F64) {
+                double d = (double)std::rand() / (double)RAND_MAX;
+                std::memcpy(&buf[i * 8], &d, 8);
+            } else if (dtype == MMBO_F16) {
                 _Float16 h = (_Float16)v;
                 std::memcpy(&buf[i * 2], &h, 2);
             } else {
@@ -71,8 +79,8 @@ int main(int argc, char **argv)
     HIP_CHECK(hipMemcpy(dC, hC.data(), hC.size(), hipMemcpyHostToDevice));
 
     auto call = [&](int id) {
-        return mmbo_gemm_strided_batched(dtype, ta, tb, M, N, K, &alpha, dA, lda, (long long)a_elems, dB, ldb,
-                                         (long long)b_elems, &beta, dC, ldc, (long long)c_elems, batch, id, NULL);
+        return mmbo_gemm_strided_batched(dtype, ta, tb, M, N, K, alpha, dA, lda, (long long)a_elems, dB, ldb,
+                                         (long long)b_elems, beta, dC, ldc, (long long)c_elems, batch, id, NULL);
     };
     auto time_config = [&](int id, float *seconds) {
         int rc = call(id);                       // warm-up, also tells whether the config applies
@@ -86,7 +94,7 @@ int main(int argc, char **argv)
         *seconds = t / reps;
         return (int)MMBO_OK;
     };
-    const char *tn = ta ? "T" : "N", *tbn = tb ? "T" : "N", *dn = dtype == MMBO_F16 ? "hgemm" : "sgemm";
+    const char *tn = ta ? "T" : "N", *tbn = tb ? "T" : "N", *dn = dtype == MMBO_F16 ? "hgemm" : dtype == MMBO_F64 ? "dgemm" : "sgemm";
     const double flops = 2.0 * (double)M * N * K * batch;
     if (type == 0) {
         int id = mmbo_select_config(dtype, ta, tb, M, N, K, batch);

@@ -6,7 +6,7 @@
 cd "$(dirname "$0")"
 mode=${1:-configs}
 if [ "$mode" = hpl ]; then
-  dt=${2:-s}
+  dt=${2:-d}
   for M in {44160..384..-3840}; do
     ./benchmark 1 ${M} 2048 384 ${M} 2048 44160 N T ${dt} 1 -1 1 || exit 1
   done
@@ -22,4 +22,5 @@ else
     ./benchmark 0 128 4096 8192 128 8192 128 N N ${dt} 1 1 0 || exit 1
   done
   ./benchmark 0 512 512 512 512 512 512 T N h 64 1 1 || exit 1
+  ./benchmark 0 44160 2048 384 44160 2048 44160 N T d 1 -1 1 || exit 1
 fi

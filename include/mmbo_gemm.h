@@ -1,5 +1,5 @@
 /*
- * mmbo_gemm.h -- C ABI of the MI355X (gfx950) SGEMM/HGEMM library.
+ * mmbo_gemm.h -- C ABI of the MI355X (gfx950) SGEMM/HGEMM/DGEMM library.
  *
  * Plain C: pointers, sizes and status codes only.  Every entry point names the piece of
  * the reference harness (CSWater/GEMM_MMBO, paths relative to its tree) that it replaces.
@@ -16,7 +16,8 @@
  *     alpha and beta are HOST pointers read before the call returns (src/gemm/gemm.h:31-32);
  *   - MMBO_F32: float A, B, C, alpha, beta; fp32 MFMA accumulate.
  *     MMBO_F16: IEEE binary16 A, B, C; alpha and beta are float; fp32 MFMA accumulate,
- *     one round-to-nearest-even to binary16 on the store;
+ *     one round-to-nearest-even to binary16 on the store.
+ *     MMBO_F64: double A, B, C, alpha, beta (the reference's own element type); fp64 MFMA accumulate;
  *   - the launch is asynchronous on `stream` (a hipStream_t, NULL = the null stream the
  *     reference uses, src/gemm/common.h:12); the caller synchronises;
  *   - config_id selects a row of the tile-config table, like the reference's kernelId
@@ -35,6 +36,7 @@ extern "C" {
 
 #define MMBO_F32 0
 #define MMBO_F16 1
+#define MMBO_F64 2
 
 #define MMBO_OP_N 0
 #define MMBO_OP_T 1
@@ -86,7 +88,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
                               int batch, int config_id, void *stream);
 
 /* Tile-config table access.  Replaces indexing the parallel arrays of src/gemm/constants.h
- * and the NUM_KERNELS sweep bound of src/gemm/benchmark.cc:10,89-109. */
+ * and the NUM_KERNELS sweep bound of src/gemm/benchmark.cc:10,89-109.  Each element type has its own
+ * table: ids are only meaningful together with the dtype they were asked for. */
 int mmbo_num_configs(int dtype);
 int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out);
 
@@ -108,7 +111,8 @@ int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm
 int mmbo_release_workspace(void);
 
 /* Measures what the MFMA pipes of the current device sustain with nothing else running: a register-only loop
- * of v_mfma_f32_32x32x16_f16 (MMBO_F16) or v_mfma_f32_32x32x2_f32 (MMBO_F32), two wavefronts per SIMD, operands
+ * of v_mfma_f32_32x32x16_f16 (MMBO_F16), v_mfma_f32_32x32x2_f32 (MMBO_F32) or v_mfma_f64_16x16x4_f64 (MMBO_F64),
+ * two wavefronts per SIMD, operands
  * all 1.0 (random_operands = 0) or uniform random (1).  Returns TFLOP/s and the average shader clock in MHz.
  * Counterpart of the reference's issue-only probe kernel src/gemm/assembly/error_kernel_000.s and of the
  * hard-coded 6.5 TFLOP/s peak its harness divides by (src/gemm/test.cc:88).  Allocates and frees a few

@@ -84,14 +84,19 @@ void oracle_f16_to_f32_array(const uint16_t *src, float *dst, size_t n)
 static inline double load_elem(int dtype, const void *p, size_t idx)
 {
     if (dtype == ORACLE_F16) return (double)oracle_f16_to_f32(((const uint16_t *)p)[idx]);
+    if (dtype == ORACLE_F64) return ((const double *)p)[idx];
     return (double)((const float *)p)[idx];
 }
 
-static inline void store_elem(int dtype, void *p, size_t idx, float v)
+/* one rounding from double to the element type */
+static inline void store_elem(int dtype, void *p, size_t idx, double v)
 {
-    if (dtype == ORACLE_F16) ((uint16_t *)p)[idx] = oracle_f32_to_f16(v);
-    else ((float *)p)[idx] = v;
+    if (dtype == ORACLE_F16) ((uint16_t *)p)[idx] = oracle_f32_to_f16((float)v);
+    else if (dtype == ORACLE_F64) ((double *)p)[idx] = v;
+    else ((float *)p)[idx] = (float)v;
 }
+
+static inline size_t elem_size(int dtype) { return dtype == ORACLE_F16 ? 2 : dtype == ORACLE_F64 ? 8 : 4; }
 
 int oracle_num_threads(void)
 {
@@ -119,7 +124,7 @@ int oracle_num_threads(void)
 static int bad_args(int dtype, int transA, int transB, size_t m, size_t n, size_t k, size_t lda,
                     size_t ldb, size_t ldc, int batch)
 {
-    if (dtype != ORACLE_F32 && dtype != ORACLE_F16) return 1;
+    if (dtype != ORACLE_F32 && dtype != ORACLE_F16 && dtype != ORACLE_F64) return 1;
     if ((transA | transB) & ~1) return 1;
     if (batch < 0) return 1;
     if (lda < (transA ? k : m) || ldb < (transB ? n : k) || ldc < m) return 1;
@@ -136,7 +141,7 @@ int oracle_gemm_f64(int dtype, int transA, int transB, size_t m, size_t n, size_
     if (bad_args(dtype, transA, transB, m, n, k, lda, ldb, ldc, batch))
         return -1;
     if (m == 0 || n == 0) return 0;
-    size_t esz = dtype == ORACLE_F16 ? 2 : 4;
+    size_t esz = elem_size(dtype);
     for (int b = 0; b < batch; ++b) {
         const char *Ab = (const char *)A + (size_t)b * (size_t)strideA * esz;
         const char *Bb = (const char *)B + (size_t)b * (size_t)strideB * esz;
@@ -161,10 +166,10 @@ int oracle_gemm_native(int dtype, int transA, int transB, size_t m, size_t n, si
                        const void *A, size_t lda, const void *B, size_t ldb, float beta, void *C,
                        size_t ldc, int batch, long long strideA, long long strideB, long long strideC)
 {
-    if (bad_args(dtype, transA, transB, m, n, k, lda, ldb, ldc, batch))
+    if (bad_args(dtype, transA, transB, m, n, k, lda, ldb, ldc, batch) || dtype == ORACLE_F64)
         return -1;
     if (m == 0 || n == 0) return 0;
-    size_t esz = dtype == ORACLE_F16 ? 2 : 4;
+    size_t esz = elem_size(dtype);
     for (int b = 0; b < batch; ++b) {
         const char *Ab = (const char *)A + (size_t)b * (size_t)strideA * esz;
         const char *Bb = (const char *)B + (size_t)b * (size_t)strideB * esz;
@@ -185,7 +190,36 @@ int oracle_gemm_native(int dtype, int transA, int transB, size_t m, size_t n, si
     return 0;
 }
 
-/* The definition, spelled out: one thread, one element at a time, ascending l. */
+/* The reference's own arithmetic: fp64 operands, fp64 multiply-add chains, C updated in place
+ * (src/gemm/gemm.h:4-5 naive_dgemm; src/gemm/ref/Kernels.cpp:84-87 with DATA_TYPE double). */
+int oracle_dgemm_native(int transA, int transB, size_t m, size_t n, size_t k, double alpha, const double *A,
+                        size_t lda, const double *B, size_t ldb, double beta, double *C, size_t ldc, int batch,
+                        long long strideA, long long strideB, long long strideC)
+{
+    if (bad_args(ORACLE_F64, transA, transB, m, n, k, lda, ldb, ldc, batch))
+        return -1;
+    if (m == 0 || n == 0) return 0;
+    for (int b = 0; b < batch; ++b) {
+        const double *Ab = A + (size_t)b * (size_t)strideA, *Bb = B + (size_t)b * (size_t)strideB;
+        double *Cb = C + (size_t)b * (size_t)strideC;
+        double *sums;
+        size_t nib;
+        if (contract_f64(ORACLE_F64, transA, transB, m, n, k, Ab, lda, Bb, ldb, &sums, &nib)) return -1;
+#pragma omp parallel for schedule(static)
+        for (size_t j = 0; j < n; ++j)
+            for (size_t i = 0; i < m; ++i) {
+                double r = alpha * sum_at_f64(sums, nib, i, j);
+                if (beta != 0.0) r = fma(beta, Cb[i + j * ldc], r);
+                Cb[i + j * ldc] = r;
+            }
+        free(sums);
+    }
+    return 0;
+}
+
+/* The definition, spelled out: one thread, one element at a time, ascending l.  For fp64 operands the
+ * sum is carried in long double (64-bit significand on x86-64), so it also bounds the rounding of the
+ * blocked fp64 contraction above. */
 int oracle_gemm_naive(int dtype, int transA, int transB, size_t m, size_t n, size_t k, double alpha,
                       const void *A, size_t lda, const void *B, size_t ldb, double beta, const void *C,
                       size_t ldc, double *out)
@@ -194,14 +228,18 @@ int oracle_gemm_naive(int dtype, int transA, int transB, size_t m, size_t n, siz
         return -1;
     for (size_t j = 0; j < n; ++j)
         for (size_t i = 0; i < m; ++i) {
-            double acc = 0.0;
+            long double acc = 0.0L;
             for (size_t l = 0; l < k; ++l) {
                 double a = load_elem(dtype, A, transA ? l + i * lda : i + l * lda);
                 double b = load_elem(dtype, B, transB ? j + l * ldb : l + j * ldb);
-                acc += a * b;
+                if (dtype == ORACLE_F64) acc += (long double)a * (long double)b;
+                else acc = (long double)((double)acc + a * b);     /* narrow operands: products are exact in double */
             }
-            out[i + j * m] = beta != 0.0 ? alpha * acc + beta * load_elem(dtype, C, i + j * ldc)
-                                         : alpha * acc;
+            long double r = (long double)alpha * acc;
+            if (beta != 0.0) r += (long double)beta * (long double)load_elem(dtype, C, i + j * ldc);
+            out[i + j * m] = dtype == ORACLE_F64 ? (double)r
+                                                 : (beta != 0.0 ? alpha * (double)acc + beta * load_elem(dtype, C, i + j * ldc)
+                                                                : alpha * (double)acc);
         }
     return 0;
 }
@@ -211,7 +249,7 @@ double oracle_max_rel_err(int dtype, const void *got, size_t ldg, long long stri
                           double *max_abs_err)
 {
     double worst = 0.0, worst_abs = 0.0;
-    size_t esz = dtype == ORACLE_F16 ? 2 : 4;
+    size_t esz = elem_size(dtype);
     for (int b = 0; b < batch; ++b) {
         const char *gb = (const char *)got + (size_t)b * (size_t)strideG * esz;
         const double *wb = want + (size_t)b * m * n;
@@ -255,7 +293,7 @@ void oracle_fill_uniform(void *dst, int dtype, size_t n, uint64_t seed, uint64_t
     for (size_t i = 0; i < n; ++i) {
         uint64_t r = oracle_rng_u64(seed, offset + i);
         double u = (double)(r >> 11) * (1.0 / 9007199254740992.0);   /* [0,1) on 53 bits */
-        store_elem(dtype, dst, i, (float)(2.0 * u - 1.0));
+        store_elem(dtype, dst, i, 2.0 * u - 1.0);
     }
 }
 
@@ -268,7 +306,7 @@ void oracle_fill_normal(void *dst, int dtype, size_t n, uint64_t seed, uint64_t 
         double u1 = ((double)(r1 >> 11) + 1.0) * (1.0 / 9007199254740992.0);   /* (0,1] */
         double u2 = (double)(r2 >> 11) * (1.0 / 9007199254740992.0);
         double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
-        store_elem(dtype, dst, i, (float)(z * scale));
+        store_elem(dtype, dst, i, z * scale);
     }
 }
 

@@ -15,7 +15,7 @@
  *   src/gemm/ref/map.cpp:7-38 and src/gemm/ref/Kernels.cpp:204-236   work-group remap (WGM)
  *   src/gemm/test.cc:39-50           fill order A, then B, then C from one random stream
  *
- * The reference computes in fp64 and only in the NT form; the four transposes,
+ * The reference computes in fp64 (ORACLE_F64 here) and only in the NT form; the four transposes,
  * fp32 and fp16 follow the BLAS definition  C = alpha*op(A)*op(B) + beta*C  with
  * op(X) = X or X^T, which is what the macros above state for op = (N, T).
  *
@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-enum { ORACLE_F32 = 0, ORACLE_F16 = 1 };   /* element type of A, B, C */
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_F64 = 2 };   /* element type of A, B, C */
 enum { ORACLE_OP_N = 0, ORACLE_OP_T = 1 };
 
 /* fp64 oracle.  out is a dense column-major m x n x batch array of doubles
@@ -59,7 +59,14 @@ int oracle_gemm_native(int dtype, int transA, int transB, size_t m, size_t n, si
                        float beta, void *C, size_t ldc,
                        int batch, long long strideA, long long strideB, long long strideC);
 
-/* Plain triple loop, fp64, no blocking, no threads: the brute-force check for the two above. */
+/* fp64 operands, fp64 chains, in place: the reference's own DGEMM arithmetic, and the timed CPU baseline of
+ * the fp64 leg.  oracle_gemm_native refuses ORACLE_F64 (its scalars are float). */
+int oracle_dgemm_native(int transA, int transB, size_t m, size_t n, size_t k, double alpha, const double *A,
+                        size_t lda, const double *B, size_t ldb, double beta, double *C, size_t ldc, int batch,
+                        long long strideA, long long strideB, long long strideC);
+
+/* Plain triple loop, no blocking, no threads: the brute-force check for the ones above.  fp32/fp16 operands
+ * are summed in fp64 (their products are exact there); fp64 operands are summed in long double. */
 int oracle_gemm_naive(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
                       double alpha, const void *A, size_t lda, const void *B, size_t ldb,
                       double beta, const void *C, size_t ldc, double *out);

@@ -14,7 +14,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-F32, F16 = 0, 1
+F32, F16, F64 = 0, 1, 2
 OP_N, OP_T = 0, 1
 
 _lib = None
@@ -39,6 +39,8 @@ def lib():
         L.oracle_gemm_native.argtypes = [ci, ci, ci, sz, sz, sz, ctypes.c_float, vp, sz, vp, sz, ctypes.c_float,
                                          vp, sz, ci, ll, ll, ll]
         L.oracle_gemm_native.restype = ci
+        L.oracle_dgemm_native.argtypes = [ci, ci, sz, sz, sz, dbl, vp, sz, vp, sz, dbl, vp, sz, ci, ll, ll, ll]
+        L.oracle_dgemm_native.restype = ci
         L.oracle_gemm_naive.argtypes = [ci, ci, ci, sz, sz, sz, dbl, vp, sz, vp, sz, dbl, vp, sz, vp]
         L.oracle_gemm_naive.restype = ci
         L.oracle_max_rel_err.argtypes = [ci, vp, sz, ll, vp, sz, sz, ci, dbl, ctypes.POINTER(dbl)]
@@ -61,7 +63,7 @@ def lib():
 
 
 def np_dtype(dtype):
-    return np.float32 if dtype == F32 else np.float16
+    return {F32: np.float32, F16: np.float16, F64: np.float64}[dtype]
 
 
 def _ptr(a):
@@ -69,7 +71,7 @@ def _ptr(a):
 
 
 def _check(a, dtype, name):
-    want = np.float32 if dtype == F32 else (np.float16, np.uint16)
+    want = np.float32 if dtype == F32 else np.float64 if dtype == F64 else (np.float16, np.uint16)
     if a.dtype not in (want if isinstance(want, tuple) else (want,)):
         raise TypeError(f"{name}: dtype {a.dtype} does not match oracle dtype {dtype}")
     if not a.flags["C_CONTIGUOUS"] and not a.flags["F_CONTIGUOUS"]:
@@ -94,6 +96,12 @@ def gemm_native(dtype, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, 
                 batch=1, strideA=0, strideB=0, strideC=0):
     """native-precision CPU GEMM, in place on C (the timed CPU baseline)."""
     _check(A, dtype, "A"); _check(B, dtype, "B"); _check(C, dtype, "C")
+    if dtype == F64:
+        rc = lib().oracle_dgemm_native(transA, transB, m, n, k, float(alpha), _ptr(A), lda, _ptr(B), ldb, float(beta),
+                                       _ptr(C), ldc, batch, strideA, strideB, strideC)
+        if rc != 0:
+            raise ValueError("oracle_dgemm_native: bad arguments")
+        return C
     rc = lib().oracle_gemm_native(dtype, transA, transB, m, n, k, float(alpha), _ptr(A), lda, _ptr(B), ldb,
                                   float(beta), _ptr(C), ldc, batch, strideA, strideB, strideC)
     if rc != 0:

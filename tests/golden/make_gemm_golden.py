@@ -3,7 +3,8 @@ matmul -- an implementation independent of oracle/host_gemm.c -- so the oracle c
 
 Inputs are drawn with numpy's own PCG64 generator (not the oracle's), rounded to the operand type, and
 stored with their leading dimensions; `want` is alpha * op(A) @ op(B) + beta * C in float64 on the
-exactly representable input values.
+exactly representable input values.  The fp64 cases (dtype code 2) are multiplied in numpy's long double
+(64-bit significand on x86-64) and the result rounded once to float64.
 
     python tests/golden/make_gemm_golden.py
 """
@@ -14,7 +15,8 @@ import numpy as np
 rng = np.random.default_rng(20240607)
 cases = {}
 idx = 0
-for dtype_name, npdt in (("f32", np.float32), ("f16", np.float16)):
+for dtype_code, npdt in ((0, np.float32), (1, np.float16), (2, np.float64)):
+    wide = np.longdouble if dtype_code == 2 else np.float64
     for ta in (0, 1):
         for tb in (0, 1):
             for (m, n, k, pad, alpha, beta) in ((5, 7, 3, 0, 1.5, 0.5), (33, 17, 41, 3, -1.0, 1.0), (64, 2, 129, 1, 1.0, 0.0)):
@@ -24,15 +26,16 @@ for dtype_name, npdt in (("f32", np.float32), ("f16", np.float16)):
                 A = rng.uniform(-1, 1, size=(lda, ac)).astype(npdt)
                 B = rng.uniform(-1, 1, size=(ldb, bc)).astype(npdt)
                 C = rng.uniform(-1, 1, size=(ldc, n)).astype(npdt)
-                opA = A[:ar, :].astype(np.float64)
+                opA = A[:ar, :].astype(wide)
                 opA = opA.T if ta else opA
-                opB = B[:br, :].astype(np.float64)
+                opB = B[:br, :].astype(wide)
                 opB = opB.T if tb else opB
                 want = alpha * (opA @ opB)
                 if beta != 0:
-                    want = want + beta * C[:m, :].astype(np.float64)
+                    want = want + beta * C[:m, :].astype(wide)
+                want = want.astype(np.float64)
                 key = f"c{idx:02d}"
-                cases[key + "_meta"] = np.array([0 if dtype_name == "f32" else 1, ta, tb, m, n, k, lda, ldb, ldc],
+                cases[key + "_meta"] = np.array([dtype_code, ta, tb, m, n, k, lda, ldb, ldc],
                                                 dtype=np.int64)
                 cases[key + "_ab"] = np.array([alpha, beta], dtype=np.float64)
                 # column-major flat buffers

@@ -6,8 +6,9 @@
 //
 //     test [M N K [transA transB dtype alpha beta kernelId]]
 //
-// Defaults follow the reference: M=44160 N=2048 K=384, NT, alpha=-1, beta=1 (src/gemm/test.cc:20-21),
-// inputs in [0,1].  Unlike the reference, which always returns 0, the exit status is 1 on a mismatch.
+// Defaults follow the reference: M=44160 N=2048 K=384, NT, fp64 (dtype d; s and h select fp32 and fp16),
+// alpha=-1, beta=1 (src/gemm/test.cc:20-21); with those defaults the call goes through naive_dgemm(), the
+// reference's own entry point.  Unlike the reference, which always returns 0, the exit status is 1 on a mismatch.
 #include <cmath>
 #include <cstring>
 #include <vector>
@@ -29,20 +30,23 @@ int main(int argc, char **argv)
     }
     const int ta = argc > 4 && (argv[4][0] == 'T' || argv[4][0] == 't');
     const int tb = argc > 5 ? (argv[5][0] == 'T' || argv[5][0] == 't') : 1;
-    const int dtype = argc > 6 && (argv[6][0] == 'h' || argv[6][0] == 'H') ? MMBO_F16 : MMBO_F32;
-    float alpha = argc > 7 ? (float)std::atof(argv[7]) : -1.0f;
-    float beta = argc > 8 ? (float)std::atof(argv[8]) : 1.0f;
+    const char dch = argc > 6 ? argv[6][0] : 'd';
+    const int dtype = (dch == 'h' || dch == 'H') ? MMBO_F16 : (dch == 's' || dch == 'S') ? MMBO_F32 : MMBO_F64;
+    const int odt = dtype == MMBO_F16 ? ORACLE_F16 : dtype == MMBO_F64 ? ORACLE_F64 : ORACLE_F32;
+    double alpha = argc > 7 ? std::atof(argv[7]) : -1.0;
+    double beta = argc > 8 ? std::atof(argv[8]) : 1.0;
+    float alpha_f = (float)alpha, beta_f = (float)beta;
     const int kernel_id = argc > 9 ? std::atoi(argv[9]) : MMBO_CONFIG_AUTO;
 
     const size_t lda = ta ? K : M, ldb = tb ? N : K, ldc = M;
     const size_t a_elems = lda * (ta ? M : K), b_elems = ldb * (tb ? K : N), c_elems = ldc * N;
-    const size_t esz = dtype == MMBO_F16 ? 2 : 4;
+    const size_t esz = dtype == MMBO_F16 ? 2 : dtype == MMBO_F64 ? 8 : 4;
     std::vector<unsigned char> A(a_elems * esz), B(b_elems * esz), C(c_elems * esz), C0(c_elems * esz);
     // seeded, in [0,1] like the reference's rand()/RAND_MAX: (uniform[-1,1) + 1) / 2 is not needed for the
     // check, so the oracle's own generator is used directly and shifted on the fly
-    oracle_fill_uniform(A.data(), dtype == MMBO_F16 ? ORACLE_F16 : ORACLE_F32, a_elems, 1, 0);
-    oracle_fill_uniform(B.data(), dtype == MMBO_F16 ? ORACLE_F16 : ORACLE_F32, b_elems, 1, a_elems);
-    oracle_fill_uniform(C.data(), dtype == MMBO_F16 ? ORACLE_F16 : ORACLE_F32, c_elems, 1, a_elems + b_elems);
+    oracle_fill_uniform(A.data(), odt, a_elems, 1, 0);
+    oracle_fill_uniform(B.data(), odt, b_elems, 1, a_elems);
+    oracle_fill_uniform(C.data(), odt, c_elems, 1, a_elems + b_elems);
 
     void *dA, *dB, *dC, *dC0;
     HIP_CHECK(hipMalloc(&dA, A.size()));
@@ -55,7 +59,12 @@ int main(int argc, char **argv)
     HIP_CHECK(hipMemcpy(dC0, C.data(), C.size(), hipMemcpyHostToDevice));
 
     auto launch = [&](void *c) {
-        return mmbo_gemm(dtype, ta, tb, M, N, K, &alpha, dA, lda, dB, ldb, &beta, c, ldc, kernel_id, NULL);
+        if (dtype == MMBO_F64 && !ta && tb)
+            return naive_dgemm(M, N, K, &alpha, (const double *)dA, lda, (const double *)dB, ldb, &beta, (double *)c, ldc,
+                               kernel_id);
+        if (dtype == MMBO_F64)
+            return mmbo_gemm(dtype, ta, tb, M, N, K, &alpha, dA, lda, dB, ldb, &beta, c, ldc, kernel_id, NULL);
+        return mmbo_gemm(dtype, ta, tb, M, N, K, &alpha_f, dA, lda, dB, ldb, &beta_f, c, ldc, kernel_id, NULL);
     };
     float elapsed = 0.0f;
     hipEvent_t e0, e1;
@@ -64,14 +73,14 @@ int main(int argc, char **argv)
     MMBO_CHECK(launch(dC0));
     GPU_TIMER_END(elapsed, e0, e1);
     const double tflops = 1e-12 * 2.0 * M * N * K / elapsed;
-    const double peak = dtype == MMBO_F16 ? 2500.0 : 157.3;
+    const double peak = dtype == MMBO_F16 ? 2500.0 : dtype == MMBO_F64 ? 78.6 : 157.3;
     std::printf("%s(%s%s): m, n, k, time, tflops, efficiency = %zu, %zu, %zu, %.5f, %.5f, %.2f%%\n",
-                dtype == MMBO_F16 ? "naive_hgemm" : "naive_sgemm", ta ? "T" : "N", tb ? "T" : "N", M, N, K, elapsed,
+                dtype == MMBO_F16 ? "naive_hgemm" : dtype == MMBO_F64 ? "naive_dgemm" : "naive_sgemm", ta ? "T" : "N", tb ? "T" : "N", M, N, K, elapsed,
                 tflops, tflops / peak * 100.0);
     HIP_CHECK(hipMemcpy(C0.data(), dC0, C0.size(), hipMemcpyDeviceToHost));
 
     std::vector<double> want(M * N);
-    if (oracle_gemm_f64(dtype == MMBO_F16 ? ORACLE_F16 : ORACLE_F32, ta, tb, M, N, K, alpha, A.data(), lda, B.data(),
+    if (oracle_gemm_f64(odt, ta, tb, M, N, K, alpha, A.data(), lda, B.data(),
                         ldb, beta, C.data(), ldc, want.data(), 1, 0, 0, 0) != 0) {
         std::fprintf(stderr, "oracle rejected the arguments\n");
         return 1;
@@ -80,11 +89,15 @@ int main(int argc, char **argv)
     for (double w : want) ss += w * w;
     const double rms = std::sqrt(ss / (double)want.size());
     double abs_err = 0.0;
-    const double rel = oracle_max_rel_err(dtype == MMBO_F16 ? ORACLE_F16 : ORACLE_F32, C0.data(), ldc, 0, want.data(),
+    const double rel = oracle_max_rel_err(odt, C0.data(), ldc, 0, want.data(),
                                           M, N, 1, rms > 0 ? rms : 1.0, &abs_err);
-    const double limit = dtype == MMBO_F16 ? 2e-2 : 1e-5 * std::sqrt((double)(K ? K : 1));
-    std::printf(" C[0][0]: %f;  oracle: %f\n", dtype == MMBO_F16 ? oracle_f16_to_f32(((uint16_t *)C0.data())[0])
-                                                                  : ((float *)C0.data())[0], want[0]);
+    const double rootk = std::sqrt((double)(K ? K : 1));
+    const double limit = dtype == MMBO_F16 ? 2e-2 : dtype == MMBO_F64 ? 2e-15 * rootk : 1e-5 * rootk;
+    std::printf(" C[0][0]: %f;  oracle: %f\n",
+                dtype == MMBO_F16   ? oracle_f16_to_f32(((uint16_t *)C0.data())[0])
+                : dtype == MMBO_F64 ? ((double *)C0.data())[0]
+                                    : ((float *)C0.data())[0],
+                want[0]);
     std::printf("max rel err %.3e (abs %.3e, rms %.3e), limit %.3e\n", rel, abs_err, rms, limit);
     const bool ok = rel <= limit;
     std::printf(ok ? "result check passed\n" : "error! result check not pass\n");

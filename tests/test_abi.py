@@ -33,9 +33,10 @@ def test_every_declared_symbol_is_exported():
 
 
 def test_config_table_rows_are_consistent():
-    for dtype in (G.F32, G.F16):
+    for dtype in (G.F32, G.F16, G.F64):
         n = G.num_configs(dtype)
-        assert n >= 6
+        assert n >= 4
+        mfma = 16 if dtype == G.F64 else 32          # MFMA block edge: 16x16x4 fp64, 32x32 otherwise
         names = set()
         for cid in range(n):
             d = G.config_info(dtype, cid)
@@ -44,7 +45,7 @@ def test_config_table_rows_are_consistent():
             assert d["macro_tile_m"] % d["wave_tile_m"] == 0 and d["macro_tile_n"] % d["wave_tile_n"] == 0
             waves = (d["macro_tile_m"] // d["wave_tile_m"]) * (d["macro_tile_n"] // d["wave_tile_n"])
             assert waves * 64 == d["threads"]
-            assert d["wave_tile_m"] % 32 == 0 and d["wave_tile_n"] % 32 == 0      # 32x32 MFMA blocks
+            assert d["wave_tile_m"] % mfma == 0 and d["wave_tile_n"] % mfma == 0
             assert 0 < d["lds_bytes"] <= 160 * 1024                                # gfx950: 160 KB per CU
             assert d["split_k"] in (1, 2, 4, 8, 16)
         assert len(names) == n
@@ -70,6 +71,10 @@ def test_select_config_headline_and_skinny_shapes():
     d = G.config_info(G.F32, G.select_config(G.F32, 0, 0, 40, 40, 64))
     assert d["macro_tile_m"] <= 64 and d["split_k"] == 1
     assert G.select_config(G.F32, 0, 0, 0, 5, 5) == 0
+    # fp64 has its own table: the reference's HPL trailing update gets a large tile, a tiny problem a small one
+    hpl = G.config_info(G.F64, G.select_config(G.F64, 0, 1, 44160, 2048, 384))
+    assert hpl["macro_tile_m"] * hpl["macro_tile_n"] >= 128 * 128 and hpl["split_k"] == 1
+    assert G.config_info(G.F64, G.select_config(G.F64, 0, 1, 40, 40, 64))["macro_tile_m"] <= 64
     with pytest.raises(G.MmboError):
         G.select_config(3, 0, 0, 1, 1, 1)
     with pytest.raises(G.MmboError):
@@ -138,6 +143,8 @@ def test_argument_validation_returns_status_codes():
     assert _call(A=None) == 4
     assert _call(cfg=10 ** 6) == 5
     assert _call(cfg=-2) == 5
+    assert _call(dtype=2, cfg=G.num_configs(G.F64)) == 5      # ids are per element type: fp64 has fewer rows
+    assert _call(dtype=2, lda=3) == 3
     # empty problems succeed without touching anything (null pointers allowed)
     assert _call(m=0, A=None, B=None, C=None, lda=1, ldc=1) == 0
     assert _call(n=0, A=None, B=None, C=None) == 0
@@ -155,5 +162,5 @@ def test_python_front_ends_keep_reference_argument_order():
     """src/gemm/gemm.h:4-5: (m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kernelId)."""
     import inspect
     want = ["m", "n", "k", "alpha", "A", "lda", "B", "ldb", "beta", "C", "ldc", "kernelId"]
-    for f in (G.naive_sgemm, G.naive_hgemm, G.sgemm_NT, G.sgemm_TN, G.hgemm_NN, G.hgemm_TT):
+    for f in (G.naive_dgemm, G.dgemm_NT, G.naive_sgemm, G.naive_hgemm, G.sgemm_NT, G.sgemm_TN, G.hgemm_NN, G.hgemm_TT):
         assert list(inspect.signature(f).parameters) == want

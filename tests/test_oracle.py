@@ -13,7 +13,7 @@ import pytest
 from oracle import oracle as O
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-F32, F16 = O.F32, O.F16
+F32, F16, F64 = O.F32, O.F16, O.F64
 
 
 # ------------------------------------------------------------------ work-group remap
@@ -107,6 +107,8 @@ def test_rng_uniform_matches_independent_numpy_restatement():
     assert got.min() >= -1.0 and got.max() < 1.0 + 1e-7
     got16 = O.fill_uniform(n, F16, seed, off)
     assert np.array_equal(got16.view(np.uint16), want.astype(np.float16).view(np.uint16))
+    got64 = O.fill_uniform(n, F64, seed, off)          # fp64 keeps all 53 bits of the draw
+    assert got64.dtype == np.float64 and np.array_equal(got64, 2.0 * u - 1.0)
 
 
 def test_rng_streams_are_position_addressed_and_distinct():
@@ -150,18 +152,19 @@ def test_oracle_against_numpy_float64_fixtures(key, z):
     Cn = C.copy()
     O.gemm_native(dtype, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, Cn, ldc)
     rel, _ = O.max_rel_err(dtype, Cn, ldc, want, m, n, floor=max(float(np.sqrt(np.mean(want ** 2))), 1e-30))
-    assert rel <= (1e-5 * np.sqrt(k) if dtype == F32 else 2e-2)
+    assert rel <= {F32: 1e-5 * np.sqrt(k), F16: 2e-2, F64: 2e-15 * np.sqrt(k)}[dtype]
     # rows m..ldc-1 of C are padding: never written
     pad_before = C.reshape((ldc, n), order="F")[m:, :]
     pad_after = Cn.reshape((ldc, n), order="F")[m:, :]
     assert np.array_equal(np.ascontiguousarray(pad_before).view(np.uint8), np.ascontiguousarray(pad_after).view(np.uint8))
 
 
-@pytest.mark.parametrize("dtype", [F32, F16])
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
 def test_blocked_equals_brute_force(dtype, ta, tb):
-    """Sizes that straddle the packing panels (8/4 rows, 4 columns) and the 512-deep k blocks."""
+    """Sizes that straddle the packing panels (8/4 rows, 4 columns) and the 512-deep k blocks.  For fp64 operands
+    the brute-force sum is carried in long double, so this also bounds the blocked fp64 sum's rounding."""
     for (m, n, k) in ((1, 1, 1), (9, 5, 3), (17, 6, 513), (40, 23, 1030)):
         ar, ac = (k, m) if ta else (m, k)
         br, bc = (n, k) if tb else (k, n)
@@ -172,7 +175,7 @@ def test_blocked_equals_brute_force(dtype, ta, tb):
         assert np.max(np.abs(fast - slow)) <= 1e-12 * max(1.0, float(np.max(np.abs(slow))))
 
 
-@pytest.mark.parametrize("dtype", [F32, F16])
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
 def test_closed_forms(dtype):
     npdt = O.np_dtype(dtype)
     m, n, k = 19, 13, 31
@@ -200,7 +203,7 @@ def test_closed_forms(dtype):
     assert np.array_equal(Cn.reshape((m, n), order="F"), exact.astype(npdt))
 
 
-@pytest.mark.parametrize("dtype", [F32, F16])
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
 def test_transpose_identity(dtype):
     """(op(A) op(B))^T = op(B)^T op(A)^T: the TN product equals the NT product of the swapped operands."""
     m, n, k = 21, 34, 55
@@ -226,6 +229,28 @@ def test_beta_zero_never_reads_c():
     assert np.all(np.isfinite(C))
     C2 = np.full(m * n, np.nan, np.float32)
     assert np.all(np.isnan(O.gemm_f64(F32, 0, 0, m, n, k, 1.0, A, m, B, k, 1.0, C2, m)))
+
+
+def test_dgemm_native_is_the_fp64_contraction_in_place():
+    """oracle_dgemm_native (the reference's own arithmetic, src/gemm/gemm.h:4-5 with alpha=-1, beta=1 as in
+    src/gemm/test.cc:20-21): equals the dense fp64 oracle, leaves padding rows alone, and is exact on integers."""
+    m, n, k, ldc = 37, 29, 61, 41
+    A, B, C = O.fill_uniform(m * k, F64, 1), O.fill_uniform(n * k, F64, 2), O.fill_uniform(ldc * n, F64, 3)
+    want = O.gemm_f64(F64, 0, 1, m, n, k, -1.0, A, m, B, n, 1.0, C, ldc)[:, :, 0]
+    Cn = C.copy()
+    O.gemm_native(F64, 0, 1, m, n, k, -1.0, A, m, B, n, 1.0, Cn, ldc)
+    got = Cn.reshape((ldc, n), order="F")
+    assert np.max(np.abs(got[:m] - want)) <= 4 * np.finfo(np.float64).eps * np.max(np.abs(want))
+    assert np.array_equal(got[m:], C.reshape((ldc, n), order="F")[m:])
+    rng = np.random.default_rng(1)
+    Ai, Bi = rng.integers(-9, 10, m * k).astype(np.float64), rng.integers(-9, 10, n * k).astype(np.float64)
+    Ci = rng.integers(-9, 10, m * n).astype(np.float64)
+    exact = -(Ai.reshape((m, k), order="F") @ Bi.reshape((n, k), order="F").T) + Ci.reshape((m, n), order="F")
+    O.gemm_native(F64, 0, 1, m, n, k, -1.0, Ai, m, Bi, n, 1.0, Ci, m)
+    assert np.array_equal(Ci.reshape((m, n), order="F"), exact)
+    # the float-scalar entry point refuses fp64 operands
+    assert O.lib().oracle_gemm_native(F64, 0, 0, 2, 2, 2, 1.0, A.ctypes.data, 2, B.ctypes.data, 2, 0.0, Cn.ctypes.data, 2,
+                                      1, 0, 0, 0) != 0
 
 
 def test_strided_batch_equals_independent_calls():

@@ -3,6 +3,8 @@ C ABI, comparison against the fp64 oracle with the tolerances the library promis
 
 Tolerances (max over C of |got - exact| / max(|exact|, rms(exact))):
     fp32:  <= 1e-5 * sqrt(K)        fp16 in/out with fp32 accumulate:  <= 2e-2
+    fp64:  <= 2e-15 * sqrt(K)  (both sides are fp64 sums of K terms in different orders; a random-walk estimate
+           of their difference is ~0.3 * 2^-53 * sqrt(K) * a few sigma, an order of magnitude below the limit)
 """
 import math
 
@@ -10,10 +12,14 @@ import numpy as np
 
 from oracle import oracle as O
 
-F32, F16 = 0, 1
+F32, F16, F64 = 0, 1, 2
+ESZ = {F32: 4, F16: 2, F64: 8}
+BITS = {F32: np.uint32, F16: np.uint16, F64: np.uint64}
 
 
 def tol(dtype, k):
+    if dtype == F64:
+        return 2e-15 * math.sqrt(max(k, 1))
     return 1e-5 * math.sqrt(max(k, 1)) if dtype == F32 else 2e-2
 
 
@@ -73,12 +79,13 @@ def run_gpu(p, config_id=-1, offset_elems=(0, 0, 0)):
     import gemm_mmbo_amd as G
 
     def up(h, off):
-        t = torch.zeros(h.size + off + 8, dtype=torch.float32 if p.dtype == F32 else torch.float16, device="cuda")
+        t = torch.zeros(h.size + off + 8, dtype={F32: torch.float32, F16: torch.float16, F64: torch.float64}[p.dtype],
+                        device="cuda")
         t[off:off + h.size].copy_(torch.from_numpy(h))
         return t
 
     dA, dB, dC = up(p.A, offset_elems[0]), up(p.B, offset_elems[1]), up(p.C, offset_elems[2])
-    esz = 4 if p.dtype == F32 else 2
+    esz = ESZ[p.dtype]
     pa = dA.data_ptr() + offset_elems[0] * esz
     pb = dB.data_ptr() + offset_elems[1] * esz
     pc = dC.data_ptr() + offset_elems[2] * esz
@@ -102,8 +109,8 @@ def check(p, got, label=""):
     limit = tol(p.dtype, p.k)
     assert rel <= limit, f"{label}: max rel err {rel:.3e} (abs {abs_err:.3e}, rms {rms:.3e}) > {limit:.3e}"
     if p.ldc > p.m:
-        g = got.view(np.uint32 if p.dtype == F32 else np.uint16)
-        c = p.C.view(np.uint32 if p.dtype == F32 else np.uint16)
+        g = got.view(BITS[p.dtype])
+        c = p.C.view(BITS[p.dtype])
         for b in range(p.batch):
             gb = g[b * p.sc: b * p.sc + p.ldc * p.n].reshape((p.ldc, p.n), order="F")
             cb = c[b * p.sc: b * p.sc + p.ldc * p.n].reshape((p.ldc, p.n), order="F")
