@@ -18,6 +18,7 @@ LIB = os.path.join(CSRC, "libmmbo_gemm.so")
 NUM_TILES = 6  # keep in step with csrc/configs.hpp
 NUM_RING_TILES = 4
 NUM_F64_TILES = 6
+NUM_X16_TILES = 5
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -37,6 +38,8 @@ def _units():
         for tile in range(NUM_RING_TILES):
             units.append(("inst_ring.hip", f"inst_ring_{dtype}_{tile}.o",
                           [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
+    for tile in range(NUM_X16_TILES):
+        units.append(("inst_x16.hip", f"inst_x16_{tile}.o", [f"-DMMBO_TILE={tile}"]))
     for tile in range(NUM_F64_TILES):
         units.append(("inst_dgemm.hip", f"inst_dgemm_{tile}.o", [f"-DMMBO_TILE={tile}"]))
     extra = os.path.join(CSRC, "extra_units.txt")

@@ -63,4 +63,15 @@ constexpr RingRow kRingTiles[NUM_RING_TILES] = {
 };
 constexpr int ring_bk(int dtype) { return dtype == 0 ? 16 : 32; }
 
+// HGEMM tiles of the 16x16x32-MFMA ring kernel with accumulation-register accumulators (hgemm_x16.hpp); depthU 32.
+// Config ids continue after the ring and wide ones:  x16_tile + NUM_X16_TILES * split_index.
+constexpr int NUM_X16_TILES = 5;
+constexpr RingRow kX16Tiles[NUM_X16_TILES] = {
+    {256, 256, 2, 2, 5},     // four wavefronts of 128 x 128: 256 accumulator registers per lane, one work-group per CU
+    {256, 256, 4, 2, 5},     // eight wavefronts of 64 x 128
+    {128, 128, 2, 2, 5},     //  80 KB of LDS, two work-groups per CU
+    {128,  64, 2, 2, 6},     //  72 KB, two per CU
+    { 64,  64, 2, 2, 6},     //  48 KB, three per CU
+};
+
 }  // namespace mmbo

@@ -43,6 +43,7 @@ struct GemmArgs {
     uint32_t k_per_split;   // multiple of the config's depthU
     uint32_t batch;
     uint32_t vec_a, vec_b, vec_c;   // 1 when 128-bit accesses to that operand are aligned
+    uint32_t chip_block;    // 1: tiles are walked in 16 x 16 chip-wide blocks (chip_block_remap) instead of wg_remap
 };
 
 // Linear work-group id -> (tile row, tile column).
@@ -71,6 +72,36 @@ __host__ __device__ inline void wg_remap(uint32_t id, uint32_t nwg0, uint32_t nw
     uint32_t width = rem == 0 ? wgm : rem;
     wg0 = serial / width;
     wg1 = serial % width + block * wgm;
+}
+
+// Linear work-group id -> (tile row, tile column) in chip-wide blocks, for a chip of 8 XCDs x 32 CUs that runs one
+// work-group per CU (the 256 x 256 tiles).
+//
+// The 256 work-groups resident at one time form one 16 x 16 block of tiles; inside it XCD x (= id % 8, the
+// dispatcher's round-robin) owns a 4 x 8 sub-block, the XCDs arranged 4 down x 2 across.  Blocks are walked down
+// the tile rows and then across, serpentine, so consecutive blocks share a panel of B.  What this buys: at
+// any moment the chip streams 16 tile rows of A and 16 tile columns of B (64 MB + 64 MB for fp16 at k = 8192), which
+// the 256 MB last-level cache holds, instead of all of A and B at once (wg_remap's order at 8192^3: 256 MB, which
+// that cache then cannot hold and every XCD's L2 misses go to HBM).  Per XCD the L2 sees the same 12 panels per
+// 32 tiles as with wg_remap.  Tiles outside the whole 16 x 16 blocks (grids that are not multiples of 16) follow
+// in column-major order.  Requires nwg0 >= 16 and nwg1 >= 16; a bijection of [0, nwg0*nwg1).
+__host__ __device__ inline void chip_block_remap(uint32_t id, uint32_t nwg0, uint32_t nwg1, uint32_t &wg0, uint32_t &wg1)
+{
+    const uint32_t f0 = nwg0 / 16, f1 = nwg1 / 16, full = f0 * f1 * 256;
+    if (id < full) {
+        const uint32_t blk = id >> 8, r = id & 255, x = r & 7, loc = r >> 3;
+        uint32_t b1 = blk / f0, b0 = blk % f0;
+        if (b1 & 1) b0 = f0 - 1 - b0;
+        wg0 = b0 * 16 + (x & 3) * 4 + (loc & 3);
+        wg1 = b1 * 16 + (x >> 2) * 8 + (loc >> 2);
+        return;
+    }
+    uint32_t rem = id - full;
+    const uint32_t w0 = nwg0 - f0 * 16, ca = f1 * 16;       // rows below the blocks, columns the blocks span
+    if (rem < w0 * ca) { wg0 = f0 * 16 + rem % w0; wg1 = rem / w0; return; }
+    rem -= w0 * ca;
+    wg0 = rem % nwg0;
+    wg1 = ca + rem / nwg0;
 }
 
 template <typename T> struct ElemTraits;

@@ -1,0 +1,445 @@
+// HGEMM ring kernel on v_mfma_f32_16x16x32_f16 with the accumulators pinned to the accumulation registers.
+//
+// Same structure as gemm_ring.hpp (whole tiles only; K in 32-wide slices through a ring of LDS buffers filled by
+// global->LDS direct loads; fragments double-buffered in registers; one barrier per slice), and the same recipe
+// as the reference's kernels (src/gemm/ref/Kernels.cpp:412-747).  Two differences, both about energy: MI355X
+// lowers its clock under the power that fp16 MFMAs on real data draw, so what a kernel costs per flop outside
+// the matrix pipe, and what the matrix instruction itself costs, decide the rate.
+//   - 16x16x32 blocks: measured on the same random operands a register-only loop of v_mfma_f32_16x16x32_f16
+//     sustains about 11 % more flop/s than one of v_mfma_f32_32x32x16_f16 (the chip holds a higher clock).
+//   - a wavefront owns up to 128 x 128 of C (256 accumulator registers per lane): four wavefronts cover a
+//     256 x 256 tile and read every LDS byte twice per slice instead of three times with eight 64 x 128 wavefronts.
+//     The accumulators live in a[0..255] by name: written by the MFMAs below, read back in the epilogue, never
+//     seen by the register allocator (left to choose, it shuttles accumulator tiles between the two register
+//     files inside the loop and spills).  Every statement that touches them lists all of them as clobbered, so
+//     the compiler neither uses them for anything else nor under-counts the kernel's registers.
+#pragma once
+
+#include "gemm_ring.hpp"
+
+namespace mmbo {
+
+namespace x16 {
+
+using ring::lds_read_b128;
+using ring::lds_read_tr16_b64;
+using ring::static_for;
+
+#define MMBO_AGPR_0_63 \
+    "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15" , \
+    "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31" , \
+    "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47" , \
+    "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63"
+#define MMBO_AGPR_64_127 \
+    "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79" , \
+    "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95" , \
+    "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111" , \
+    "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127"
+#define MMBO_AGPR_128_255 \
+    "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143" , \
+    "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159" , \
+    "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175" , \
+    "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191" , \
+    "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207" , \
+    "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223" , \
+    "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239" , \
+    "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
+
+// acc block BASE/4 += A-fragment x B-fragment.  NACC = accumulator registers the kernel owns (64, 128 or 256).
+template <int BASE, int NACC>
+__device__ __forceinline__ void mfma_acc(const u32x4 &a, const u32x4 &b)
+{
+    static_assert(BASE % 4 == 0 && BASE + 4 <= NACC, "accumulator block out of range");
+    if constexpr (NACC > 128)
+        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
+    else if constexpr (NACC > 64)
+        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
+    else
+        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63);
+}
+template <int NACC>
+__device__ __forceinline__ void acc_zero()
+{
+    static_for<NACC>([&](auto I) {
+        if constexpr (NACC > 128)
+            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
+        else if constexpr (NACC > 64)
+            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
+        else
+            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63);
+    });
+    asm volatile("s_nop 7" ::: "memory");
+}
+template <int I>
+__device__ __forceinline__ float acc_read()
+{
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(I));
+    return x;
+}
+
+// One operand tile of one slice: R rows x 32 k = R * 64 bytes, fetched by NW wavefronts with 1 KB direct loads.
+//   KC (source contiguous along k): LDS row r = its 64 bytes; 16-byte chunk c sits at position c ^ ((r >> 1) & 3).
+//     A fragment read (ds_read_b128, lane l -> row l % 16, chunk l / 16) was timed on MI355X with candidate
+//     swizzles: this one runs at the conflict-free rate, the ring kernel's (r >> 2) & 3 at half of it for this
+//     lane pattern (and at the full rate for the ring kernel's own row l % 32, chunk l / 32).
+//   RC (source contiguous along the row index): LDS k-row = R halves.  A transposing read takes, per 16-lane
+//     block, four consecutive k-rows x 32 bytes; its blocks sit 8 k-rows apart.  The chunk index is XORed with a
+//     mask of k so that the four k-rows of a block fall into different 64-byte groups and the two blocks served
+//     in one pass into different halves of a group.
+template <bool KC, int R, int NW>
+struct Tile {
+    static constexpr int BYTES = R * 64;
+    static constexpr int INSTRS = R / 16;
+    static_assert(INSTRS % NW == 0, "tile must split evenly over the wavefronts");
+    static constexpr int LPW = INSTRS / NW;
+    static constexpr int ROW_BYTES = R * 2;
+    static constexpr int CPR = ROW_BYTES / 16;
+    static constexpr int KPI = 1024 / ROW_BYTES;
+    static_assert(KC || R == 64 || R == 128 || R == 256, "RC tile: a k-row is 128, 256 or 512 bytes");
+
+    __device__ static inline uint32_t rc_mask(uint32_t k)
+    {
+        if constexpr (ROW_BYTES % 256 == 0) return ((k & 3) << 2) | (((k >> 3) & 1) << 1);
+        else return (((k >> 1) & 1) << 2) | (((k >> 3) & 1) << 1);    // 128-byte k-rows alternate between bank halves
+    }
+    __device__ static inline uint32_t kc_swz(uint32_t row) { return (row >> 1) & 3; }
+    __device__ static inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ kc_swz(row)) << 4); }
+    __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4); }
+
+    // global byte offset (from the tile origin of this slice) of the chunk that lands in LDS slot (wave*LPW + i)*64 + lane
+    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld)
+    {
+        const uint32_t q = wave * LPW + i;
+        if constexpr (KC) {
+            uint32_t row = q * 16 + (lane >> 2);
+            uint32_t chunk = (lane & 3) ^ kc_swz(row);
+            return row * ld * 2 + chunk * 16;
+        } else {
+            uint32_t k = q * KPI + lane / CPR;
+            uint32_t chunk = (lane % CPR) ^ rc_mask(k);
+            return k * ld * 2 + chunk * 16;
+        }
+    }
+};
+
+// Fragments of one operand of one wavefront for one slice: F blocks of 16 rows x 32 k, four registers each.
+// Lane l holds row l % 16, k = (l / 16) * 8 + 0..7 -- the operand layout of the 16x16x32 MFMA, for both operands.
+template <bool KC, int R, int NW, int F>
+struct Frags {
+    using T = Tile<KC, R, NW>;
+    static constexpr int RPF = KC ? 1 : 2;          // LDS reads per fragment
+    static constexpr int NOPS = F * RPF;
+    u32x4 x[F];
+
+    struct Addr { uint32_t a[KC ? 1 : F]; };
+
+    __device__ static inline Addr make_addr(int lane, int r0)
+    {
+        Addr ad;
+        if constexpr (KC) {
+            ad.a[0] = T::kc_off(r0 + (lane & 15), lane >> 4);                     // + f*16*64 per block
+        } else {
+            // transposing read: lane j of a 16-lane block points at k-row j/4, rows 4*(j%4)..+3, and receives
+            // (k-rows 0..3) x (row j); block b covers k = 8b + 4h + 0..3 with its h-th read
+            const uint32_t j = lane & 15, b = lane >> 4;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                uint32_t m = r0 + f * 16 + (j & 3) * 4;
+                uint32_t k = b * 8 + (j >> 2);                                    // + 4h: not in the swizzle mask
+                ad.a[f] = T::rc_off(k, m >> 3) + (m & 7) * 2;
+            }
+        }
+        return ad;
+    }
+
+    template <int OP>
+    __device__ __forceinline__ void read_op(uint32_t tile, const Addr &ad)
+    {
+        constexpr int f = OP / RPF, h = OP % RPF;
+        if constexpr (KC) {
+            x[f] = lds_read_b128<f * 16 * 64>(tile + ad.a[0]);
+        } else {
+            u32x2 v = lds_read_tr16_b64<h * 4 * T::ROW_BYTES>(tile + ad.a[f]);
+            x[f][2 * h] = v[0];
+            x[f][2 * h + 1] = v[1];
+        }
+    }
+    __device__ __forceinline__ void read_all(uint32_t tile, const Addr &ad)
+    {
+        static_for<NOPS>([&](auto OP) { this->template read_op<decltype(OP)::value>(tile, ad); });
+    }
+};
+
+}  // namespace x16
+
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
+struct X16Cfg {
+    static constexpr int NW = WM * WN, NT = NW * 64;
+    static constexpr int BK = 32;
+    static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 16, FN = TN / 16;
+    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA block");
+    static constexpr int NACC = FM * FN * 4 > 128 ? 256 : FM * FN * 4 > 64 ? 128 : 64;    // accumulation registers claimed
+    static_assert(FM * FN * 4 <= 256, "wave tile needs more than 256 accumulator registers");
+    using TileA = x16::Tile<TA, BM, NW>;
+    using TileB = x16::Tile<!TB, BN, NW>;
+    using FragA = x16::Frags<TA, BM, NW, FM>;
+    using FragB = x16::Frags<!TB, BN, NW, FN>;
+    static constexpr int SLICE_BYTES = TileA::BYTES + TileB::BYTES;
+    static constexpr int LDS_BYTES = DEPTH * SLICE_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "ring does not fit the 160 KB of LDS");
+    static constexpr int BATCH = TileA::LPW + TileB::LPW;         // direct loads per thread per slice
+    static constexpr int NMFMA = FM * FN;
+    static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
+};
+
+// ABLATE: timing probe as in gemm_ring.hpp (bit 0 no direct loads, bit 1 no LDS reads, bit 2 no MFMAs); results
+// are wrong by design and the library only instantiates ABLATE = 0.
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+__global__ void __launch_bounds__(WM * WN * 64)
+hgemm_x16_kernel(const GemmArgs args)
+{
+    using namespace x16;
+    using Cfg = X16Cfg<TA, TB, BM, BN, WM, WN, DEPTH>;
+    using TileA = typename Cfg::TileA;
+    using TileB = typename Cfg::TileB;
+    using FragA = typename Cfg::FragA;
+    using FragB = typename Cfg::FragB;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC;
+
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wn = wave / WM;
+
+    uint32_t wg0, wg1;
+    if (args.chip_block) chip_block_remap(blockIdx.x, args.nwg0, args.nwg1, wg0, wg1);
+    else wg_remap(blockIdx.x, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
+    const uint32_t zb = blockIdx.z;
+    const uint32_t split = zb / args.batch, batch = zb % args.batch;
+    const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
+    const uint32_t lda = args.lda, ldb = args.ldb;
+    const uint32_t k_begin = split * args.k_per_split;
+    const uint32_t k_end = min(args.k, k_begin + args.k_per_split);
+    const int n_slice = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
+
+    const char *gA = static_cast<const char *>(args.A) +
+                     ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda + k_begin
+                                                          : (int64_t)k_begin * lda + row0)) * 2;
+    const char *gB = static_cast<const char *>(args.B) +
+                     ((int64_t)batch * args.strideB + (TB ? (int64_t)k_begin * ldb + col0
+                                                          : (int64_t)col0 * ldb + k_begin)) * 2;
+    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * 2;
+    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * 2;
+
+    uint32_t offA[TileA::LPW], offB[TileB::LPW];
+#pragma unroll
+    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda);
+#pragma unroll
+    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb);
+
+    // direct load number l (A's first, then B's) of slice s into ring buffer `buf`
+    auto issue_load = [&](auto L, const char *pa, const char *pb, char *dst) {
+        constexpr int l = decltype(L)::value;
+        if constexpr (l < TileA::LPW)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pa + offA[l]),
+                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + l) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pb + offB[l - TileA::LPW]),
+                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024), 16, 0, 0);
+    };
+    auto issue_slice = [&](int s, int buf) {
+        if constexpr (ABLATE & 1) return;
+        char *dst = lds + buf * Cfg::SLICE_BYTES;
+        const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
+        static_for<BATCH>([&](auto L) { issue_load(L, pa, pb, dst); });
+    };
+
+    const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
+    const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
+    FragA fa[2];
+    FragB fb[2];
+    if constexpr (ABLATE != 0) {      // the probes' MFMAs must see operand bits like the real ones: power depends on them
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(args.A);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+#pragma unroll
+            for (int f = 0; f < FM; ++f) fa[q].x[f] = src[(q * 16 + f) * 64 + lane];
+#pragma unroll
+            for (int f = 0; f < FN; ++f) fb[q].x[f] = src[(q * 16 + 8 + f) * 64 + lane];
+        }
+    }
+
+    acc_zero<NACC>();
+
+    const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
+    auto read_slice = [&](FragA &a, FragB &b, int buf) {
+        if constexpr (ABLATE & 2) return;
+        const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
+        a.read_all(t, adA);
+        b.read_all(t + TileA::BYTES, adB);
+    };
+
+    // One slice: its MFMAs from register set (ca, cb), with the LDS reads of the next slice (into na, nb) issued
+    // between the first READ_SPAN of them and this wavefront's direct loads of slice s+DEPTH spread over all of
+    // them.  A wavefront issues in order and here it is alone on its SIMD: memory instructions issued as a block
+    // would stall the matrix pipe behind the LDS / texture-address queues, and reads issued late would leave their
+    // latency exposed before the barrier.
+    constexpr int NA = FragA::NOPS, NR = FragA::NOPS + FragB::NOPS, NMFMA = Cfg::NMFMA;
+    constexpr int READ_SPAN = Cfg::NW > 4 ? NMFMA : NMFMA * 3 / 4;     // two wavefronts per SIMD cover each other's read latency
+    auto mfma_and_read = [&](auto LOAD, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
+        constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load`
+        const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
+        char *dst = lds + lbuf * Cfg::SLICE_BYTES;
+        const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
+        static_for<NMFMA>([&](auto M) {
+            constexpr int m = decltype(M)::value;
+            // boustrophedon over the FM x FN blocks: consecutive MFMAs share one operand register, also at the row
+            // ends (a register-only loop of these MFMAs runs 3 % faster when one operand repeats than when both change)
+            constexpr int i = m / FN, j = (i & 1) ? FN - 1 - m % FN : m % FN;
+            if constexpr (!(ABLATE & 4)) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (!(ABLATE & 2) && m < READ_SPAN) {
+                constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
+                static_for<r1 - r0>([&](auto RR) {
+                    constexpr int r = r0 + decltype(RR)::value;
+                    if constexpr (r < NA) na.template read_op<r>(t, adA);
+                    else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
+                });
+            }
+            if constexpr (!(ABLATE & 1) && load_mode != 0) {
+                // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
+                constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
+                static_for<l1 - l0>([&](auto LL) {
+                    constexpr int l = l0 + decltype(LL)::value;
+                    if constexpr (l < BATCH) {
+                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, pa, pb, dst);
+                    }
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+#define MMBO_BARRIER()                           \
+    do {                                         \
+        __builtin_amdgcn_sched_barrier(0);       \
+        __builtin_amdgcn_s_barrier();            \
+        __builtin_amdgcn_sched_barrier(0);       \
+    } while (0)
+#define MMBO_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+#define MMBO_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
+
+    // Without the MFMAs nothing reads the fragments, and a register whose asynchronous LDS read is still in flight
+    // could be handed to something else (a load address, say) before the data lands in it: keep them live past the wait.
+    auto keep_alive = [&](const FragA &a, const FragB &b) {
+        if constexpr ((ABLATE & 4) != 0) {
+#pragma unroll
+            for (int f = 0; f < FM; ++f) asm volatile("" :: "v"(a.x[f]));
+#pragma unroll
+            for (int f = 0; f < FN; ++f) asm volatile("" :: "v"(b.x[f]));
+        }
+    };
+
+    // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
+    // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free; this
+    // wavefront's loads of slices s+2 .. s+DEPTH-1 are in flight.  Loads return in order, so waiting for all but the
+    // newest DEPTH-2 batches means this wavefront's part of slice s+2 has landed.
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s)
+        if (s < n_slice) issue_slice(s, s);
+    if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
+    MMBO_BARRIER();                                                  // slice 0 resident
+    read_slice(fa[0], fb[0], 0);
+    MMBO_WAIT_LGKM0();
+    keep_alive(fa[0], fb[0]);
+    if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
+    MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
+
+    int buf = 0;                                                     // s % DEPTH
+    // steady state: every slice issues loads, no flag tests inside the MFMA stream
+    auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+        const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+        mfma_and_read(std::integral_constant<int, 1>{}, ca, cb, na, nb, nbuf, true, s + DEPTH, buf);
+        MMBO_WAIT_LGKM0();
+        keep_alive(na, nb);
+        MMBO_WAIT_VM(BATCH * (DEPTH - 2));
+        MMBO_BARRIER();
+        buf = nbuf;
+    };
+    // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
+    // interleaved block free of divergent control flow)
+    auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+        const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+        const bool load = s + DEPTH < n_slice;
+        mfma_and_read(std::integral_constant<int, 2>{}, ca, cb, na, nb, nbuf, load, s + DEPTH, buf);
+        MMBO_WAIT_LGKM0();
+        keep_alive(na, nb);
+        if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();
+        buf = nbuf;
+    };
+    int s = 0;
+    for (; s + 1 + DEPTH < n_slice; s += 2) {
+        steady_step(s, fa[0], fb[0], fa[1], fb[1]);
+        steady_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+    }
+    for (; s < n_slice; s += 2) {
+        tail_step(s, fa[0], fb[0], fa[1], fb[1]);
+        if (s + 1 < n_slice) tail_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+    }
+#undef MMBO_BARRIER
+#undef MMBO_WAIT_VM
+#undef MMBO_WAIT_LGKM0
+
+    // the last MFMAs' results must have landed before they are read back
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // Epilogue.  Block (i, j): lane l holds C(row, col) for row = i*16 + 4*(l/16) + 0..3, col = j*16 + l%16 (the
+    // 16x16 MFMA result layout: four consecutive rows of one column).  C = alpha*acc (+ beta*C), the old C read only
+    // when beta != 0 (reference: src/gemm/ref/Kernels.cpp:87); with GlobalSplitU > 1 the raw sums go to the fp32
+    // workspace [split][batch][n][m] and the reduction kernel applies alpha and beta.
+    const uint32_t wrow0 = row0 + wm * Cfg::TM + 4 * (lane >> 4), wcol0 = col0 + wn * Cfg::TN + (lane & 15);
+    if (args.splits > 1) {
+        float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)args.m * args.n;
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int i = decltype(IJ)::value / FN, j = decltype(IJ)::value % FN, base = (i * FN + j) * 4;
+            float *p = ws + (size_t)(wcol0 + j * 16) * args.m + wrow0 + i * 16;
+            *reinterpret_cast<f32x4 *>(p) = f32x4{acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
+        });
+        return;
+    }
+    const float alpha = args.alpha, beta = args.beta;
+    const uint32_t ldc = args.ldc;
+    half_t *C = static_cast<half_t *>(args.C) + (int64_t)batch * args.strideC;
+    const bool vec_c = args.vec_c != 0;
+    static_for<FM * FN>([&](auto IJ) {
+        constexpr int i = decltype(IJ)::value / FN, j = decltype(IJ)::value % FN, base = (i * FN + j) * 4;
+        half_t *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
+        float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
+        if (vec_c) {
+            union { half_t e[4]; u32x2 v2; } io;
+            if (beta != 0.0f) {
+                io.v2 = *reinterpret_cast<const u32x2 *>(p);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) io.e[r] = (half_t)v[r];
+            *reinterpret_cast<u32x2 *>(p) = io.v2;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float o = v[r];
+                if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
+                p[r] = (half_t)o;
+            }
+        }
+    });
+}
+
+}  // namespace mmbo

@@ -23,20 +23,25 @@ namespace {
 constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
 constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
 constexpr int kWideConfig = kStagedConfigs + kRingConfigs;      // HGEMM NN/TT 256x256 ring with 64-k units
-constexpr int kNumConfigs = kWideConfig + 1;
+constexpr int kX16Base = kWideConfig + 1;                      // HGEMM 16x16x32-MFMA ring, (x16 tile, split) pairs
+constexpr int kX16Configs = NUM_X16_TILES * NUM_SPLITS;
+constexpr int kNumConfigs = kX16Base + kX16Configs;
 
 struct ConfigRef {
-    bool ring;
+    bool ring;      // a whole-tile kernel (ring, wide or x16): no edge handling
     int tile;
     int split;
+    bool x16;
 };
 inline ConfigRef config_ref(int id)
 {
-    if (id == kWideConfig) return {true, 0, 1};                 // same tile and grid as ring tile 0, no split
-    if (id < kStagedConfigs) return {false, id % NUM_TILES, kSplits[id / NUM_TILES]};
+    if (id >= kX16Base) return {true, (id - kX16Base) % NUM_X16_TILES, kSplits[(id - kX16Base) / NUM_X16_TILES], true};
+    if (id == kWideConfig) return {true, 0, 1, false};          // same tile and grid as ring tile 0, no split
+    if (id < kStagedConfigs) return {false, id % NUM_TILES, kSplits[id / NUM_TILES], false};
     id -= kStagedConfigs;
-    return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES]};
+    return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES], false};
 }
+inline int x16_config_id(int tile, int split_index) { return kX16Base + tile + NUM_X16_TILES * split_index; }
 inline bool valid_dtype(int dtype) { return dtype == MMBO_F32 || dtype == MMBO_F16 || dtype == MMBO_F64; }
 inline int ring_config_id(int tile, int split_index) { return kStagedConfigs + tile + NUM_RING_TILES * split_index; }
 
@@ -45,9 +50,9 @@ inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_
     return dtype == MMBO_F16 && transA == transB && m % 256 == 0 && n % 256 == 0 && k % 64 == 0 && k >= 512;
 }
 
-inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k)
+inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k, bool x16 = false)
 {
-    const RingRow &r = kRingTiles[tile];
+    const RingRow &r = x16 ? kX16Tiles[tile] : kRingTiles[tile];
     const size_t bk = (size_t)ring_bk(dtype);
     if (m % r.bm || n % r.bn || k == 0 || k % bk) return false;
     return (k / bk) % (size_t)split == 0;          // every split gets the same whole number of slices
@@ -113,6 +118,14 @@ hipError_t dispatch_ring(int tile, int ta, int tb, const GemmArgs &a, hipStream_
 {
     if (tile == TILE) return launch_ring<DTYPE, TILE>(ta, tb, a, s);
     if constexpr (TILE + 1 < NUM_RING_TILES) return dispatch_ring<DTYPE, TILE + 1>(tile, ta, tb, a, s);
+    return hipErrorInvalidValue;
+}
+
+template <int TILE>
+hipError_t dispatch_x16(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
+{
+    if (tile == TILE) return launch_x16<TILE>(ta, tb, a, s);
+    if constexpr (TILE + 1 < NUM_X16_TILES) return dispatch_x16<TILE + 1>(tile, ta, tb, a, s);
     return hipErrorInvalidValue;
 }
 
@@ -278,9 +291,10 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
         return MMBO_OK;
     }
     if (c.ring) {
-        const RingRow &r = kRingTiles[c.tile];
-        std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d", r.bm, r.bn,
-                      ring_bk(dtype), r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, c.split, r.depth);
+        const RingRow &r = c.x16 ? kX16Tiles[c.tile] : kRingTiles[c.tile];
+        std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d%s", r.bm, r.bn,
+                      ring_bk(dtype), r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, c.split, r.depth,
+                      c.x16 ? "_MFMA16x16x32_ACC" : "");
         out->macro_tile_m = r.bm;
         out->macro_tile_n = r.bn;
         out->depth_u = ring_bk(dtype);
@@ -341,18 +355,19 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         }
     }
     // ring configs: same tile geometry, deeper prefetch, no edge handling.  Where one applies it replaces the
-    // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).
+    // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).  For fp16 the ring
+    // kernel on 16x16x32 MFMAs takes its place (faster than both the 32x32x16 ring and the wide-unit kernel on every
+    // shape swept).
     {
         const ConfigRef c = config_ref(best);
         const TileRow &t = tile_row(dtype, c.tile);
+        static const int x16_of_ring[NUM_RING_TILES] = {0, 2, 3, 4};       // same macro tile in kX16Tiles (256 x 256: four wavefronts)
         for (int rt = 0; rt < NUM_RING_TILES; ++rt) {
             const RingRow &r = kRingTiles[rt];
             if (r.bm * r.bn > t.bm * t.bn) continue;
             for (int si = 0; si < NUM_SPLITS; ++si)
-                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k)) {
-                    if (rt == 0 && si == 0 && wide_ok(dtype, transA, transB, m, n, k)) return kWideConfig;
-                    return ring_config_id(rt, si);
-                }
+                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k))
+                    return dtype == MMBO_F16 ? x16_config_id(x16_of_ring[rt], si) : ring_config_id(rt, si);
         }
     }
     return best;
@@ -366,6 +381,18 @@ int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm
     if ((unsigned long long)nwg0 * nwg1 > 0xFFFFFFFFull || linear_id >= nwg0 * nwg1) return MMBO_ERR_INVALID_SIZE;
     uint32_t a, b;
     wg_remap(linear_id, nwg0, nwg1, wgm, num_xcd, a, b);
+    *wg0 = a;
+    *wg1 = b;
+    return MMBO_OK;
+}
+
+int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned *wg0, unsigned *wg1)
+{
+    if (!wg0 || !wg1) return MMBO_ERR_NULL_POINTER;
+    if (nwg0 < 16 || nwg1 < 16) return MMBO_ERR_INVALID_SIZE;
+    if ((unsigned long long)nwg0 * nwg1 > 0xFFFFFFFFull || linear_id >= nwg0 * nwg1) return MMBO_ERR_INVALID_SIZE;
+    uint32_t a, b;
+    chip_block_remap(linear_id, nwg0, nwg1, a, b);
     *wg0 = a;
     *wg1 = b;
     return MMBO_OK;
@@ -426,11 +453,12 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     const ConfigRef cref = f64 ? ConfigRef{false, config_id, 1} : config_ref(config_id);
     const size_t esz = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
     int split = cref.split;
-    TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{kRingTiles[cref.tile].bm, kRingTiles[cref.tile].bn, ring_bk(dtype), 0, 0}
-                          : tile_row(dtype, cref.tile);
-    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
+    const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
+    TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0} : tile_row(dtype, cref.tile);
+    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
+    if (cref.x16 && dtype != MMBO_F16) return MMBO_ERR_INVALID_CONFIG;
 
     // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
     {
@@ -463,6 +491,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     a.splits = (uint32_t)split;
     a.k_per_split = (uint32_t)(split > 1 ? k_per_split : (k ? k : 1));
     a.batch = (uint32_t)batch;
+    a.chip_block = cref.x16 && r.bm == 256 && r.bn == 256 && nwg0 >= 16 && nwg1 >= 16;
     auto aligned16 = [&](const void *p, size_t ld, long long stride) {
         return ((uintptr_t)p % 16 == 0) && ((ld * esz) % 16 == 0) && (((size_t)stride * esz) % 16 == 0);
     };
@@ -480,6 +509,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     hipError_t e;
     if (f64) e = dispatch_dgemm<0>(cref.tile, transA, transB, a, s);
     else if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
+    else if (cref.x16) e = dispatch_x16<0>(cref.tile, transA, transB, a, s);
     else if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
                                          : dispatch_ring<1, 0>(cref.tile, transA, transB, a, s);
     else e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(cref.tile, transA, transB, a, s)

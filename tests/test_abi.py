@@ -112,6 +112,40 @@ def test_wg_remap_groups_each_xcd_on_neighbouring_tiles():
         assert len(cols) <= 8 and len(rows) <= 5
 
 
+@pytest.mark.parametrize("nwg0,nwg1", [(32, 32), (16, 16), (17, 16), (16, 19), (35, 50), (48, 33)])
+def test_chip_block_remap_bijection_and_block_structure(nwg0, nwg1):
+    """The chip-wide block order of the 256 x 256 HGEMM tiles: a bijection; every run of 256 consecutive ids inside
+    the whole blocks covers exactly one 16 x 16 block of tiles, and the 32 ids of one XCD (id % 8) in it a 4 x 8
+    sub-block; consecutive blocks share their tile rows or their tile columns (one operand panel stays cached)."""
+    seen = set()
+    tiles = [G.chip_block_remap(lid, nwg0, nwg1) for lid in range(nwg0 * nwg1)]
+    for t in tiles:
+        assert 0 <= t[0] < nwg0 and 0 <= t[1] < nwg1
+        seen.add(t)
+    assert len(seen) == nwg0 * nwg1
+    nblk = (nwg0 // 16) * (nwg1 // 16)
+    prev = None
+    for b in range(nblk):
+        blk = tiles[256 * b:256 * (b + 1)]
+        r0, c0 = min(t[0] for t in blk), min(t[1] for t in blk)
+        assert r0 % 16 == 0 and c0 % 16 == 0
+        assert {(t[0] - r0, t[1] - c0) for t in blk} == {(i, j) for i in range(16) for j in range(16)}
+        for x in range(8):
+            sub = blk[x::8]
+            assert max(t[0] for t in sub) - min(t[0] for t in sub) == 3
+            assert max(t[1] for t in sub) - min(t[1] for t in sub) == 7
+        if prev is not None:
+            assert prev[0] == r0 or prev[1] == c0
+        prev = (r0, c0)
+
+
+def test_chip_block_remap_rejects_bad_arguments():
+    with pytest.raises(G.MmboError):
+        G.chip_block_remap(0, 15, 16)        # fewer than 16 tile rows
+    with pytest.raises(G.MmboError):
+        G.chip_block_remap(16 * 16, 16, 16)  # id out of range
+
+
 def test_wg_remap_rejects_bad_arguments():
     with pytest.raises(G.MmboError):
         G.wg_remap(10, 2, 5, 8, 8)          # id out of range

@@ -91,7 +91,8 @@ def test_every_config_aligned_interior(dtype):
     import gemm_mmbo_amd as G
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
-        if dtype == F32 and "+3U" in G.config_info(dtype, cid)["name"]:      # an fp16-only kernel
+        name = G.config_info(dtype, cid)["name"]
+        if dtype == F32 and ("+3U" in name or "MFMA16x16x32" in name):      # fp16-only kernels
             with pytest.raises(G.MmboError):
                 U.run_gpu(p, cid)
             continue
@@ -99,25 +100,36 @@ def test_every_config_aligned_interior(dtype):
 
 
 def _ring_ids(dtype):
+    """Config ids of the generic direct-to-LDS ring kernel (32x32 MFMA blocks)."""
     import gemm_mmbo_amd as G
-    return [c for c in range(G.num_configs(dtype))
-            if "DTL1" in G.config_info(dtype, c)["name"] and "+3U" not in G.config_info(dtype, c)["name"]]
+    names = {c: G.config_info(dtype, c)["name"] for c in range(G.num_configs(dtype))}
+    return [c for c, nm in names.items() if "DTL1" in nm and "+3U" not in nm and "MFMA16x16x32" not in nm]
+
+
+def _x16_ids():
+    """Config ids of the HGEMM ring kernel on 16x16x32 MFMAs with accumulation-register accumulators."""
+    import gemm_mmbo_amd as G
+    return [c for c in range(G.num_configs(F16)) if "MFMA16x16x32" in G.config_info(F16, c)["name"]]
+
+
+def _wide_id():
+    import gemm_mmbo_amd as G
+    (cid,) = [c for c in range(G.num_configs(F16)) if "+3U" in G.config_info(F16, c)["name"]]
+    return cid
 
 
 def test_wide_unit_ring_kernel_nn_tt():
-    """The HGEMM NN/TT variant that fetches the k-contiguous operand in 64-k units (last config id): K from the
+    """The HGEMM NN/TT variant that fetches the k-contiguous operand in 64-k units: K from the
     shortest it takes (512) up, unit counts that are and are not multiples of the three unit buffers, beta, batches;
     refused for NT/TN, fp32, short or odd K."""
     import gemm_mmbo_amd as G
-    cid = G.num_configs(F16) - 1
-    assert "+3U" in G.config_info(F16, cid)["name"]
+    cid = _wide_id()
     for (ta, tb) in ((0, 0), (1, 1)):
         for (m, n, k, alpha, beta, batch) in ((256, 256, 512, 1.0, 0.0, 1), (512, 256, 576, 1.5, 0.5, 1), (256, 768, 1024, -1.0, 1.0, 2),
                                               (768, 512, 4096, 1.0, 0.0, 1), (256, 256, 640, 1.0, 0.0, 1), (256, 512, 704, 1.0, 1.0, 1)):
             p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=90 + k, dist="normal",
                           c_fill="uniform" if beta else "nan")
             _run_and_check(p, cid, label=f"wide {m}x{n}x{k}")
-        assert G.select_config(F16, ta, tb, 8192, 8192, 8192) == cid
     for (dtype, ta, tb, k) in ((F16, 0, 1, 1024), (F16, 1, 0, 1024), (F32, 0, 0, 1024), (F16, 0, 0, 448), (F16, 0, 0, 1056)):
         p = U.Problem(dtype, ta, tb, 256, 256, k, 1.0, 0.0, seed=3, c_fill="nan")
         with pytest.raises(G.MmboError) as e:
@@ -147,6 +159,54 @@ def test_ring_kernel_every_config_every_transpose(dtype, ta, tb):
             _run_and_check(p, cid, label=f"{d['name']} {m}x{n}x{k} b{batch}")
             ran += 1
     assert ran == 80
+
+
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_x16_kernel_every_config_every_transpose(ta, tb):
+    """The HGEMM ring kernel on v_mfma_f32_16x16x32_f16 with accumulators pinned to the accumulation registers, by
+    explicit config id: every tile (4 and 8 wavefronts, 64 to 256 accumulator registers) and split-K factor, K
+    shorter and longer than the ring, odd slice counts, beta read-modify-write, batches."""
+    import gemm_mmbo_amd as G
+    ids = _x16_ids()
+    assert len(ids) == 25
+    ran = 0
+    for cid in ids:
+        d = G.config_info(F16, cid)
+        assert d["depth_u"] == 32
+        bm, bn, sp = d["macro_tile_m"], d["macro_tile_n"], d["split_k"]
+        for (tm, tn, slices, alpha, beta, batch) in ((1, 1, 1, 1.0, 0.0, 1), (2, 1, 3, 1.5, 0.5, 1), (1, 3, 7, -1.0, 1.0, 2),
+                                                     (3, 2, 33, 1.0, 0.0, 1)):
+            m, n, k = bm * tm, bn * tn, 32 * slices * sp
+            p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=170 + cid + slices, dist="normal",
+                          c_fill="uniform" if beta else "nan")
+            _run_and_check(p, cid, label=f"{d['name']} {m}x{n}x{k} b{batch}")
+            ran += 1
+    assert ran == 100
+
+
+def test_x16_kernel_chip_block_order_and_refusals():
+    """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
+    ragged border of tiles, against the oracle.  Ragged shapes, fp32 and unaligned operands are refused; ld > dim and
+    the automatic pick work."""
+    import gemm_mmbo_amd as G
+    ids = _x16_ids()
+    for cid in ids[:2]:
+        assert G.config_info(F16, cid)["macro_tile_m"] == 256
+        for (m, n, k) in ((4096, 4096, 64), (4352, 4096, 96), (4096, 4608, 64), (8192, 4352, 32)):
+            p = U.Problem(F16, 0, 0, m, n, k, 1.0, 0.0, seed=300 + m // 256, dist="normal", c_fill="nan")
+            _run_and_check(p, cid, label=f"chip blocks {m}x{n}x{k}")
+    cid = ids[0]
+    for (dtype, m, n, k, offs) in ((F16, 255, 256, 128, (0, 0, 0)), (F16, 256, 300, 128, (0, 0, 0)), (F16, 256, 256, 136, (0, 0, 0)),
+                                   (F16, 256, 256, 128, (1, 0, 0)), (F32, 256, 256, 128, (0, 0, 0))):
+        p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
+        with pytest.raises(G.MmboError) as e:
+            U.run_gpu(p, cid, offs)
+        assert e.value.status == 5
+    p = U.Problem(F16, 1, 0, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71, dist="normal")
+    _run_and_check(p, cid, label="x16 ld>dim")
+    assert G.select_config(F16, 0, 0, 8192, 8192, 8192) in ids
+    assert G.select_config(F16, 0, 1, 2048, 2048, 2048) in ids
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
