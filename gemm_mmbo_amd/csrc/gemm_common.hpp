@@ -141,9 +141,9 @@ __device__ inline void write_back(const f32x16 (&acc)[FM][FN], const GemmArgs &a
     if (args.splits > 1) {
         float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)m * n;
 #pragma unroll
-        for (int i = 0; i < FM; ++i)
+        for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
+            for (int i = 0; i < FM; ++i) {
                 uint32_t col = wcol0 + j * 32 + cl;
                 if (!INTERIOR && col >= n) continue;
 #pragma unroll
@@ -167,10 +167,11 @@ __device__ inline void write_back(const f32x16 (&acc)[FM][FN], const GemmArgs &a
     const uint32_t ldc = args.ldc;
     T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
     const bool vec_c = args.vec_c != 0;
+    // down a column first: the stores that complete one cache line of C follow each other
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+    for (int j = 0; j < FN; ++j)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
+        for (int i = 0; i < FM; ++i) {
             uint32_t col = wcol0 + j * 32 + cl;
             if (!INTERIOR && col >= n) continue;
 #pragma unroll

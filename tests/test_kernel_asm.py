@@ -1,0 +1,143 @@
+"""Static checks on the gfx950 assembly hipcc generates for the direct-to-LDS kernels (no GPU needed).
+
+The ring kernels issue their LDS fragment reads as inline assembly and retire them with an explicit
+`s_waitcnt lgkmcnt(0)`: the compiler does not know that a destination register is not yet valid between the read
+and that wait.  If it ever handed such a register to something else (a copy, an address computation), the kernel
+would compute with, or load from, garbage -- a timing probe variant of the kernel once faulted exactly that way.
+These tests compile every instantiation the library ships to assembly and check, per kernel:
+
+  * no instruction between an LDS read and the next `s_waitcnt lgkmcnt(0)` names a register the read writes;
+  * nothing is spilled to scratch memory;
+  * the 16x16x32 kernel claims exactly the accumulation registers its MFMAs name (64, 128 or 256), so none of
+    them can be given to another value.
+"""
+import os
+import re
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "gemm_mmbo_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument", "--cuda-device-only", "-S"]
+
+pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
+
+#        source file            defines
+UNITS = [("inst_x16.hip", ["-DMMBO_TILE=%d" % t]) for t in range(5)] + \
+        [("inst_ring.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(4)] + \
+        [("inst_ring_wide.hip", [])]
+
+
+def _compile(unit, outdir):
+    src, defs = unit
+    out = os.path.join(outdir, src.replace(".hip", "") + "".join(d.replace("-D", "_").replace("=", "") for d in defs) + ".s")
+    r = subprocess.run([HIPCC] + FLAGS + defs + [os.path.join(CSRC, src), "-o", out], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    return out
+
+
+def _kernels(path):
+    """{kernel symbol: list of instruction lines} of one assembly file."""
+    lines = open(path).read().split("\n")
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
+    out = {}
+    for n, i in enumerate(starts):
+        end = starts[n + 1] if n + 1 < len(starts) else len(lines)
+        body = []
+        for l in lines[i + 1:end]:
+            t = l.strip()
+            if t.startswith(".amdhsa_kernel") or t.startswith(".section"):
+                break
+            if t and not t.startswith(";") and not t.startswith("."):
+                body.append(t.split(";")[0].strip())
+        out[lines[i].split(":")[0]] = body
+    return out
+
+
+def _vregs(text):
+    regs = set()
+    for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(a) for a in re.findall(r"\bv(\d+)\b", text))
+    return regs
+
+
+def _inflight_violations(body):
+    pending, bad = set(), []
+    for t in body:
+        m = re.match(r"ds_read\w* (v\[\d+:\d+\]|v\d+),", t)
+        if m:
+            addr = _vregs(t[m.end():])
+            if addr & pending:
+                bad.append(t)
+            pending |= _vregs(m.group(1))
+            continue
+        if t.startswith("s_waitcnt") and "lgkmcnt(0)" in t:
+            pending = set()
+            continue
+        if pending and (_vregs(t) & pending):
+            bad.append(t)
+    return bad
+
+
+@pytest.fixture(scope="module")
+def asm_files(tmp_path_factory):
+    outdir = str(tmp_path_factory.mktemp("asm"))
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
+        return list(ex.map(lambda u: _compile(u, outdir), UNITS))
+
+
+def test_checker_sees_a_planted_violation():
+    body = ["ds_read_b128 v[10:13], v5 offset:64", "v_add_u32_e32 v11, s3, v9", "s_waitcnt lgkmcnt(0)"]
+    assert _inflight_violations(body) == ["v_add_u32_e32 v11, s3, v9"]
+    ok = ["ds_read_b64_tr_b16 v[10:11], v5", "v_mfma_f32_16x16x32_f16 a[0:3], v[20:23], v[24:27], a[0:3]",
+          "s_waitcnt vmcnt(2)", "s_waitcnt lgkmcnt(0)", "v_mfma_f32_16x16x32_f16 a[0:3], v[10:13], v[24:27], a[0:3]"]
+    assert _inflight_violations(ok) == []
+
+
+def test_no_register_is_touched_while_its_lds_read_is_in_flight(asm_files):
+    checked = 0
+    for path in asm_files:
+        for name, body in _kernels(path).items():
+            if not any(t.startswith("ds_read") for t in body):
+                continue
+            bad = _inflight_violations(body)
+            assert not bad, f"{name}: {bad[:3]}"
+            checked += 1
+    assert checked >= 4 * (5 + 8) + 2      # four transposes of every tile, both wide kernels
+
+
+def test_no_scratch_spills(asm_files):
+    for path in asm_files:
+        for name, body in _kernels(path).items():
+            assert not any(t.startswith("scratch_") for t in body), f"{name} spills to scratch"
+
+
+def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
+    seen = 0
+    for path in asm_files:
+        if "inst_x16" not in path:
+            continue
+        text = open(path).read()
+        for name, body in _kernels(path).items():
+            used = set()
+            for t in body:
+                # (the assembler prints register indices above 64 in hex)
+                for a, b in re.findall(r"\ba\[(\w+):(\w+)\]", t):
+                    used.update(range(int(a, 0), int(b, 0) + 1))
+                used.update(int(a, 0) for a in re.findall(r"\ba\[(\w+)\]", t))
+                # no accumulation register may appear outside the MFMAs, the zeroing and the read-back
+                if re.search(r"\ba\[?\d", t):
+                    assert t.startswith(("v_mfma_f32_16x16x32_f16", "v_accvgpr_write_b32", "v_accvgpr_read_b32")), (name, t)
+            m = re.search(r"\.amdhsa_kernel " + re.escape(name) + r"\b.*?\.amdhsa_next_free_vgpr (\d+).*?\.amdhsa_accum_offset (\d+)",
+                          text, re.S)
+            assert m, name
+            agprs = int(m.group(1)) - int(m.group(2))       # registers past the unified file's accumulation offset
+            assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
+            assert agprs == len(used), (name, agprs, len(used))
+            seen += 1
+    assert seen == 20
