@@ -198,7 +198,12 @@ struct X16Cfg {
 
 // ABLATE: timing probe as in gemm_ring.hpp (bit 0 no direct loads, bit 1 no LDS reads, bit 2 no MFMAs); results
 // are wrong by design and the library only instantiates ABLATE = 0.
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+// PAIR: fetch two slices of one operand per iteration (see mfma_and_read); on when an operand is k-contiguous.
+// EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
+// unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
+// one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0, bool PAIR = (TA || !TB),
+          int EVEN_OP = (TA ? 0 : 1)>
 __global__ void __launch_bounds__(WM * WN * 64)
 hgemm_x16_kernel(const GemmArgs args)
 {
@@ -260,6 +265,18 @@ hgemm_x16_kernel(const GemmArgs args)
         static_for<BATCH>([&](auto L) { issue_load(L, pa, pb, dst); });
     };
 
+    // load number i of operand OP (0 = A, 1 = B) of slice s into ring buffer b
+    auto issue_op_load = [&](auto OP, auto I, int s, int b) {
+        constexpr int op = decltype(OP)::value, i = decltype(I)::value;
+        char *dst = lds + b * Cfg::SLICE_BYTES;
+        if constexpr (op == 0)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gA + (int64_t)s * stepA + offA[i]),
+                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + i) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gB + (int64_t)s * stepB + offB[i]),
+                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024), 16, 0, 0);
+    };
+
     const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
     const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
     FragA fa[2];
@@ -292,8 +309,18 @@ hgemm_x16_kernel(const GemmArgs args)
     // latency exposed before the barrier.
     constexpr int NA = FragA::NOPS, NR = FragA::NOPS + FragB::NOPS, NMFMA = Cfg::NMFMA;
     constexpr int READ_SPAN = Cfg::NW > 4 ? NMFMA : NMFMA * 3 / 4;     // two wavefronts per SIMD cover each other's read latency
-    auto mfma_and_read = [&](auto LOAD, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
-        constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load`
+    // Paired mode (PAIR): iteration s fetches TWO slices, s+DEPTH-1 and s+DEPTH, of ONE operand -- A on even s, B on
+    // odd s -- and issues the two loads that cover the two halves of the same 128-byte memory lines back to back.
+    // With 64-byte LDS rows a k-contiguous operand otherwise asks for every cache line twice, a slice time apart
+    // (measured: half-line requests stream at 35-52 B/clk/CU from L2, whole lines at 72-91).  `load` / `load2`
+    // say whether the first / second slice of the pair exists.
+    auto mfma_and_read = [&](auto LOAD, auto PAR, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load,
+                             bool load2, int ls, int lbuf) {
+        constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load` (and `load2`)
+        constexpr int par = decltype(PAR)::value;
+        constexpr int opn = par ^ EVEN_OP;                         // paired mode: the operand this iteration fetches
+        constexpr int LOP = opn == 0 ? TileA::LPW : TileB::LPW;   // and its loads per slice
+        const int pbuf = lbuf == 0 ? DEPTH - 1 : lbuf - 1;        // buffer of slice s+DEPTH-1
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         char *dst = lds + lbuf * Cfg::SLICE_BYTES;
         const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
@@ -312,7 +339,17 @@ hgemm_x16_kernel(const GemmArgs args)
                     else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
-            if constexpr (!(ABLATE & 1) && load_mode != 0) {
+            if constexpr (!(ABLATE & 1) && load_mode != 0 && PAIR) {
+                constexpr int l0 = (2 * LOP * m + NMFMA) / (2 * NMFMA), l1 = (2 * LOP * (m + 1) + NMFMA) / (2 * NMFMA);
+                static_for<l1 - l0>([&](auto LL) {
+                    constexpr int l = l0 + decltype(LL)::value;
+                    if constexpr (l < LOP) {
+                        if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, ls - 1, pbuf);
+                        if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, ls, lbuf);
+                    }
+                });
+            }
+            if constexpr (!(ABLATE & 1) && load_mode != 0 && !PAIR) {
                 // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
                 constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
                 static_for<l1 - l0>([&](auto LL) {
@@ -346,51 +383,132 @@ hgemm_x16_kernel(const GemmArgs args)
     };
 
     // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
-    // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free; this
-    // wavefront's loads of slices s+2 .. s+DEPTH-1 are in flight.  Loads return in order, so waiting for all but the
-    // newest DEPTH-2 batches means this wavefront's part of slice s+2 has landed.
-#pragma unroll
-    for (int s = 0; s < DEPTH; ++s)
-        if (s < n_slice) issue_slice(s, s);
-    if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
-    MMBO_BARRIER();                                                  // slice 0 resident
-    read_slice(fa[0], fb[0], 0);
-    MMBO_WAIT_LGKM0();
-    keep_alive(fa[0], fb[0]);
-    if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
-    MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
-
+    // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free (and, for the
+    // operand whose turn it is in paired mode, buffer (s-1) % DEPTH too); the loads of the later slices are in flight.
+    // Loads return in order.  Unpaired: waiting for all but the newest DEPTH-2 batches means this wavefront's part of
+    // slice s+2 has landed.  Paired: everything issued in the last DEPTH-3 iterations belongs to slices >= s+3, so all but
+    // that may stay in flight.
     int buf = 0;                                                     // s % DEPTH
-    // steady state: every slice issues loads, no flag tests inside the MFMA stream
-    auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
-        const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-        mfma_and_read(std::integral_constant<int, 1>{}, ca, cb, na, nb, nbuf, true, s + DEPTH, buf);
-        MMBO_WAIT_LGKM0();
-        keep_alive(na, nb);
-        MMBO_WAIT_VM(BATCH * (DEPTH - 2));
-        MMBO_BARRIER();
-        buf = nbuf;
-    };
-    // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
-    // interleaved block free of divergent control flow)
-    auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
-        const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-        const bool load = s + DEPTH < n_slice;
-        mfma_and_read(std::integral_constant<int, 2>{}, ca, cb, na, nb, nbuf, load, s + DEPTH, buf);
-        MMBO_WAIT_LGKM0();
-        keep_alive(na, nb);
-        if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
-        MMBO_BARRIER();
-        buf = nbuf;
-    };
     int s = 0;
-    for (; s + 1 + DEPTH < n_slice; s += 2) {
-        steady_step(s, fa[0], fb[0], fa[1], fb[1]);
-        steady_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
-    }
-    for (; s < n_slice; s += 2) {
-        tail_step(s, fa[0], fb[0], fa[1], fb[1]);
-        if (s + 1 < n_slice) tail_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+    if constexpr (!PAIR) {
+#pragma unroll
+        for (int q = 0; q < DEPTH; ++q)
+            if (q < n_slice) issue_slice(q, q);
+        if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();                                                  // slice 0 resident
+        read_slice(fa[0], fb[0], 0);
+        MMBO_WAIT_LGKM0();
+        keep_alive(fa[0], fb[0]);
+        if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
+
+        // steady state: every slice issues loads, no flag tests inside the MFMA stream
+        auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+            const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+            mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
+            MMBO_WAIT_LGKM0();
+            keep_alive(na, nb);
+            MMBO_WAIT_VM(BATCH * (DEPTH - 2));
+            MMBO_BARRIER();
+            buf = nbuf;
+        };
+        // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
+        // interleaved block free of divergent control flow)
+        auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+            const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+            const bool load = s + DEPTH < n_slice;
+            mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, s + DEPTH, buf);
+            MMBO_WAIT_LGKM0();
+            keep_alive(na, nb);
+            if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
+            MMBO_BARRIER();
+            buf = nbuf;
+        };
+        for (; s + 1 + DEPTH < n_slice; s += 2) {
+            steady_step(s, fa[0], fb[0], fa[1], fb[1]);
+            steady_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+        }
+        for (; s < n_slice; s += 2) {
+            tail_step(s, fa[0], fb[0], fa[1], fb[1]);
+            if (s + 1 < n_slice) tail_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+        }
+    } else {
+        static_assert(!PAIR || DEPTH >= 5, "paired loads need a ring of at least five buffers");
+        // X = the operand even iterations fetch (EVEN_OP), Y = the other
+        constexpr int LA = EVEN_OP == 0 ? TileA::LPW : TileB::LPW, LB = EVEN_OP == 0 ? TileB::LPW : TileA::LPW;
+        constexpr std::integral_constant<int, EVEN_OP> OPX{};
+        constexpr std::integral_constant<int, 1 - EVEN_OP> OPY{};
+        // prologue: X slices 0 .. DEPTH-2, Y slices 0 .. DEPTH-1, slice by slice (iteration 0 brings X's DEPTH-1 and DEPTH)
+        if constexpr (!(ABLATE & 1)) {
+#pragma unroll
+            for (int q = 0; q < DEPTH; ++q) {
+                if (q < n_slice) {
+                    if (q < DEPTH - 1) static_for<LA>([&](auto I) { issue_op_load(OPX, I, q, q); });
+                    static_for<LB>([&](auto I) { issue_op_load(OPY, I, q, q); });
+                }
+            }
+        }
+        constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
+        if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - BATCH); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();                                                  // slice 0 resident
+        read_slice(fa[0], fb[0], 0);
+        MMBO_WAIT_LGKM0();
+        keep_alive(fa[0], fb[0]);
+        if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - 2 * BATCH); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
+
+        // loads a steady iteration of parity P leaves in flight: those of the last DEPTH-3 iterations, itself included
+        auto steady_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+            constexpr int par = decltype(PAR)::value;
+            constexpr int own = 2 * (par == 0 ? LA : LB), other = 2 * (par == 0 ? LB : LA);
+            constexpr int KEEP = own * ((DEPTH - 3 + 1) / 2) + other * ((DEPTH - 3) / 2);
+            static_assert(KEEP < 64, "more loads in flight than vmcnt can count");
+            const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+            mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
+            MMBO_WAIT_LGKM0();
+            keep_alive(na, nb);
+            MMBO_WAIT_VM(KEEP);
+            MMBO_BARRIER();
+            buf = nbuf;
+        };
+        // tail: count what was actually issued; hist[0] is the previous iteration, hist[1] the one before
+        int hist[2] = {0, 0};
+        auto tail_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+            constexpr int par = decltype(PAR)::value;
+            constexpr int LOP = par == 0 ? LA : LB;
+            constexpr int G = LA < LB ? LA : LB;                         // every count below is a multiple of the smaller LPW
+            static_assert(LA % G == 0 && LB % G == 0, "loads per slice of one operand must divide the other's");
+            const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+            const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
+            mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, s + DEPTH, buf);
+            MMBO_WAIT_LGKM0();
+            keep_alive(na, nb);
+            const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP;
+            const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
+            constexpr int KMAX = 2 * (LA > LB ? LA : LB) * 3;
+            bool waited = false;
+            static_for<KMAX / G>([&](auto Q) {
+                constexpr int c = KMAX - decltype(Q)::value * G;          // KMAX, KMAX-G, ..., G
+                if (!waited && keep >= c) { MMBO_WAIT_VM(c); waited = true; }
+            });
+            if (!waited) MMBO_WAIT_VM(0);
+            MMBO_BARRIER();
+            hist[1] = hist[0];
+            hist[0] = cur;
+            buf = nbuf;
+        };
+        constexpr std::integral_constant<int, 0> EVEN{};
+        constexpr std::integral_constant<int, 1> ODD{};
+        for (; s + 1 + DEPTH < n_slice; s += 2) {
+            steady_step(EVEN, s, fa[0], fb[0], fa[1], fb[1]);
+            steady_step(ODD, s + 1, fa[1], fb[1], fa[0], fb[0]);
+            hist[0] = 2 * LB;
+            hist[1] = 2 * LA;
+        }
+        for (; s < n_slice; s += 2) {
+            tail_step(EVEN, s, fa[0], fb[0], fa[1], fb[1]);
+            if (s + 1 < n_slice) tail_step(ODD, s + 1, fa[1], fb[1], fa[0], fb[0]);
+        }
     }
 #undef MMBO_BARRIER
 #undef MMBO_WAIT_VM
