@@ -538,17 +538,33 @@ hgemm_x16_kernel(const GemmArgs args)
     const uint32_t ldc = args.ldc;
     half_t *C = static_cast<half_t *>(args.C) + (int64_t)batch * args.strideC;
     const bool vec_c = args.vec_c != 0;
+    if (vec_c && beta != 0.0f) {
+        // beta != 0 (reference: the fma(C, beta, .) epilogue, MT192x096x08 kernel :3037-3056): all of the wave tile's old C
+        // is requested before the first value is used -- up to 128 registers, free now that the fragments are dead -- so the
+        // read-modify-write runs at memory bandwidth instead of one load latency per block.
+        u32x2 cold[FM * FN];
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM;
+            cold[decltype(IJ)::value] = *reinterpret_cast<const u32x2 *>(C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16);
+        });
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
+            half_t *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
+            union { half_t e[4]; u32x2 v2; } io;
+            io.v2 = cold[decltype(IJ)::value];
+            float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) io.e[r] = (half_t)__builtin_fmaf(beta, (float)io.e[r], v[r]);
+            *reinterpret_cast<u32x2 *>(p) = io.v2;
+        });
+        return;
+    }
     static_for<FM * FN>([&](auto IJ) {
         constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
         half_t *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
         float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
         if (vec_c) {
             union { half_t e[4]; u32x2 v2; } io;
-            if (beta != 0.0f) {
-                io.v2 = *reinterpret_cast<const u32x2 *>(p);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
-            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) io.e[r] = (half_t)v[r];
             *reinterpret_cast<u32x2 *>(p) = io.v2;
