@@ -182,18 +182,25 @@ __device__ inline void write_back(const f32x16 (&acc)[FM][FN], const GemmArgs &a
                 float v[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * q + r];
-                if (vec_c && (INTERIOR || row + 4 <= m)) {
+                if (INTERIOR || row + 4 <= m) {
+                    // four rows in range: one vector access, aligned or not (unaligned global access is enabled
+                    // on gfx950 under ROCm; an odd ldc costs split lines, not four scalar accesses)
+                    typedef u32x4 __attribute__((aligned(4))) u32x4_u;
+                    typedef u32x2 __attribute__((aligned(2))) u32x2_u;
                     union { T e[4]; u32x4 v4; u32x2 v2; } io;
                     if (beta != 0.0f) {                       // beta == 0: C is never read
-                        if constexpr (ESZ == 4) io.v4 = *reinterpret_cast<const u32x4 *>(p);
-                        else io.v2 = *reinterpret_cast<const u32x2 *>(p);
+                        if constexpr (ESZ == 4) io.v4 = vec_c ? *reinterpret_cast<const u32x4 *>(p) : *reinterpret_cast<const u32x4_u *>(p);
+                        else io.v2 = vec_c ? *reinterpret_cast<const u32x2 *>(p) : *reinterpret_cast<const u32x2_u *>(p);
 #pragma unroll
                         for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, (float)io.e[r], v[r]);
                     }
 #pragma unroll
                     for (int r = 0; r < 4; ++r) io.e[r] = (T)v[r];
-                    if constexpr (ESZ == 4) *reinterpret_cast<u32x4 *>(p) = io.v4;
-                    else *reinterpret_cast<u32x2 *>(p) = io.v2;
+                    if constexpr (ESZ == 4) {
+                        if (vec_c) *reinterpret_cast<u32x4 *>(p) = io.v4; else *reinterpret_cast<u32x4_u *>(p) = io.v4;
+                    } else {
+                        if (vec_c) *reinterpret_cast<u32x2 *>(p) = io.v2; else *reinterpret_cast<u32x2_u *>(p) = io.v2;
+                    }
                 } else {
 #pragma unroll
                     for (int r = 0; r < 4; ++r)

@@ -56,8 +56,11 @@ struct OperandTile {
         for (int c = 0; c < NCH; ++c) regs[c] = *reinterpret_cast<const u32x4 *>(g + off[c]);
     }
 
-    // Edge tile, K tail or unaligned operand: element loads, zero where row >= rows or k >= kvalid.
-    // Whole in-range chunks still use one 128-bit load when `vec` says the operand is aligned.
+    // Edge tile, K tail or unaligned operand: zero where row >= rows or k >= kvalid.  Whole in-range chunks still
+    // use one 128-bit load, aligned or not (gfx950 under ROCm runs with unaligned global access enabled: a leading
+    // dimension like 1023 costs split cache-line accesses, not eight 2-byte loads per chunk); only chunks that
+    // straddle the matrix edge or the end of K go element by element.
+    typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;
     __device__ static inline void load_slow(u32x4 (&regs)[NCH], const char *g, const uint32_t (&off)[NCH],
                                             int tid, uint32_t ld, int rows, int kvalid, bool vec)
     {
@@ -69,6 +72,8 @@ struct OperandTile {
             bool full = row0 + nrow <= rows && k0 + nk <= kvalid;
             if (full && vec) {
                 regs[c] = *reinterpret_cast<const u32x4 *>(g + off[c]);
+            } else if (full) {
+                regs[c] = *reinterpret_cast<const u32x4_unaligned *>(g + off[c]);
             } else {
                 union { u32x4 v; T e[VEC]; } u;
                 u.v = u32x4{0, 0, 0, 0};
@@ -159,6 +164,17 @@ struct StagedCfg {
     static constexpr int LDS_BYTES = 2 * STAGE_BYTES;       // double buffer
 };
 
+// How many stages ahead the global loads run (a ring of register sets).  One stage costs a full memory latency
+// when nothing overlaps it, so short-K problems on small tiles -- few stages, little MFMA work per stage -- want
+// several in flight; the large tiles spend their registers on accumulators and keep one.
+template <typename T, int BM, int BN, int BK, int NT>
+constexpr int staged_prefetch()
+{
+    // registers per thread per stage: 4 per 128-bit chunk
+    const int regs = 4 * (BM + BN) * BK / (16 / (int)sizeof(T)) / NT;
+    return regs <= 16 ? 3 : regs <= 32 && BM * BN <= 128 * 128 ? 2 : 1;
+}
+
 template <typename T, bool TA, bool TB, int BM, int BN, int BK, int WM, int WN>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_staged_kernel(const GemmArgs args)
@@ -169,6 +185,7 @@ gemm_staged_kernel(const GemmArgs args)
     using Tr = ElemTraits<T>;
     constexpr int NT = Cfg::NT, FM = Cfg::FM, FN = Cfg::FN, ESZ = sizeof(T);
     constexpr int NKG = BK / Tr::KG;
+    constexpr int PF = staged_prefetch<T, BM, BN, BK, NT>();
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -212,17 +229,17 @@ gemm_staged_kernel(const GemmArgs args)
     // whole-tile-in-range and aligned: every stage but the K tail takes the unpredicated loader
     const bool fast = rows_a == BM && rows_b == BN && args.vec_a && args.vec_b;
 
-    u32x4 ra[TileA::NCH], rb[TileB::NCH];
-    auto load_stage = [&](int it) {
+    u32x4 ra[PF][TileA::NCH], rb[PF][TileB::NCH];             // register ring: stage `it` lives in set it % PF
+    auto load_stage = [&](int it, u32x4 (&xa)[TileA::NCH], u32x4 (&xb)[TileB::NCH]) {
         const char *pa = gA + (int64_t)it * stepA;
         const char *pb = gB + (int64_t)it * stepB;
         if (fast && it < n_full) {
-            TileA::load_fast(ra, pa, offA);
-            TileB::load_fast(rb, pb, offB);
+            TileA::load_fast(xa, pa, offA);
+            TileB::load_fast(xb, pb, offB);
         } else {
             int kvalid = it < n_full ? BK : k_tail;
-            TileA::load_slow(ra, pa, offA, tid, lda, rows_a, kvalid, args.vec_a != 0);
-            TileB::load_slow(rb, pb, offB, tid, ldb, rows_b, kvalid, args.vec_b != 0);
+            TileA::load_slow(xa, pa, offA, tid, lda, rows_a, kvalid, args.vec_a != 0);
+            TileB::load_slow(xb, pb, offB, tid, ldb, rows_b, kvalid, args.vec_b != 0);
         }
     };
 
@@ -237,17 +254,22 @@ gemm_staged_kernel(const GemmArgs args)
     const uint32_t fa_off = frag_lane_off<T, TA, TileA::LDS_LD>(lane, wm * Cfg::TM);
     const uint32_t fb_off = frag_lane_off<T, !TB, TileB::LDS_LD>(lane, wn * Cfg::TN) + TileA::LDS_BYTES;
 
+    // prologue: stages 0 .. PF-1 requested, stage 0 moved into LDS buffer 0
+#pragma unroll
+    for (int q = 0; q < PF; ++q)
+        if (q < n_iter) load_stage(q, ra[q], rb[q]);
     if (n_iter > 0) {
-        load_stage(0);
-        TileA::store_lds(ra, lds, tid);
-        TileB::store_lds(rb, lds + TileA::LDS_BYTES, tid);
+        TileA::store_lds(ra[0], lds, tid);
+        TileB::store_lds(rb[0], lds + TileA::LDS_BYTES, tid);
     }
     __syncthreads();
 
     int cur = 0;
-    for (int it = 0; it < n_iter; ++it) {
-        const bool more = it + 1 < n_iter;
-        if (more) load_stage(it + 1);                        // global prefetch of the next stage
+    // Iteration `it` (register set q = it % PF, a compile-time index inside the PF-fold unrolled body): request
+    // stage it+PF into set q, whose stage `it` already sits in LDS; multiply stage `it` from LDS buffer `cur`; move
+    // stage it+1 (set (q+1) % PF, requested PF-1 iterations ago) into the other LDS buffer; one barrier.
+    auto body = [&](int it, u32x4 (&qa)[TileA::NCH], u32x4 (&qb)[TileB::NCH], u32x4 (&na)[TileA::NCH], u32x4 (&nb)[TileB::NCH]) {
+        if (it + PF < n_iter) load_stage(it + PF, qa, qb);
 
         const char *st = lds + cur * Cfg::STAGE_BYTES;
 #pragma unroll
@@ -263,13 +285,43 @@ gemm_staged_kernel(const GemmArgs args)
                 for (int j = 0; j < FN; ++j) mma(acc[i][j], fa[i], fb[j]);
         }
 
-        if (more) {
+        if (it + 1 < n_iter) {
             char *nx = lds + (cur ^ 1) * Cfg::STAGE_BYTES;   // nobody reads this buffer during stage `it`
-            TileA::store_lds(ra, nx, tid);
-            TileB::store_lds(rb, nx + TileA::LDS_BYTES, tid);
+            TileA::store_lds(na, nx, tid);
+            TileB::store_lds(nb, nx + TileA::LDS_BYTES, tid);
         }
         __syncthreads();
         cur ^= 1;
+    };
+    for (int it0 = 0; it0 < n_iter; it0 += PF) {
+        if constexpr (PF == 1) {
+            // one set: stage it+1 is requested into it before the multiply and stored after it
+            if (it0 + 1 < n_iter) load_stage(it0 + 1, ra[0], rb[0]);
+            const char *st = lds + cur * Cfg::STAGE_BYTES;
+#pragma unroll
+            for (int kg = 0; kg < NKG; ++kg) {
+                Frag<T> fa[FM], fb[FN];
+#pragma unroll
+                for (int i = 0; i < FM; ++i) fa[i] = read_frag<T, TA, TileA::LDS_LD>(st, fa_off, i, kg);
+#pragma unroll
+                for (int j = 0; j < FN; ++j) fb[j] = read_frag<T, !TB, TileB::LDS_LD>(st, fb_off, j, kg);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j) mma(acc[i][j], fa[i], fb[j]);
+            }
+            if (it0 + 1 < n_iter) {
+                char *nx = lds + (cur ^ 1) * Cfg::STAGE_BYTES;
+                TileA::store_lds(ra[0], nx, tid);
+                TileB::store_lds(rb[0], nx + TileA::LDS_BYTES, tid);
+            }
+            __syncthreads();
+            cur ^= 1;
+        } else {
+#pragma unroll
+            for (int q = 0; q < PF; ++q)
+                if (it0 + q < n_iter) body(it0 + q, ra[q], rb[q], ra[(q + 1) % PF], rb[(q + 1) % PF]);
+        }
     }
 
     write_back<T, FM, FN, false>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, split, lane);

@@ -21,8 +21,8 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 1024, 1024, 1024, 1, 4, 75.4f},
     {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
     {0, 1, 0, 4096, 4096, 4096, 1, 30, 137.1f},
-    {0, 0, 0, 1023, 777, 513, 1, 10, 24.5f},
-    {1, 0, 0, 1023, 777, 513, 1, 10, 25.8f},
+    {0, 0, 0, 1023, 777, 513, 1, 10, 30.0f},
+    {1, 0, 0, 1023, 777, 513, 1, 10, 39.0f},
     {0, 0, 0, 4096, 128, 4096, 1, 22, 85.8f},
     {1, 0, 0, 4096, 128, 4096, 1, 64, 257.7f},
     {0, 0, 0, 128, 4096, 8192, 1, 47, 100.1f},
