@@ -18,19 +18,19 @@ struct TunedRow {
 
 constexpr TunedRow kTuned[] = {
     //dtype ta tb m n k batch id TFLOP/s
-    {0, 0, 0, 1024, 1024, 1024, 1, 4, 75.4f},
+    {0, 0, 0, 1024, 1024, 1024, 1, 33, 93.0f},
     {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
     {0, 1, 0, 4096, 4096, 4096, 1, 30, 137.1f},
     {0, 0, 0, 1023, 777, 513, 1, 10, 30.0f},
     {1, 0, 0, 1023, 777, 513, 1, 10, 39.0f},
-    {0, 0, 0, 4096, 128, 4096, 1, 22, 85.8f},
+    {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
     {1, 0, 0, 4096, 128, 4096, 1, 64, 257.7f},
     {0, 0, 0, 128, 4096, 8192, 1, 47, 100.1f},
     {1, 0, 0, 128, 4096, 8192, 1, 64, 398.7f},
     {1, 1, 0, 512, 512, 512, 64, 52, 452.0f},
-    {0, 0, 0, 2048, 2048, 2048, 1, 3, 112.0f},
+    {0, 0, 0, 2048, 2048, 2048, 1, 31, 121.0f},
     {1, 0, 0, 2048, 2048, 2048, 1, 53, 761.2f},
-    {0, 0, 1, 44160, 2048, 384, 1, 2, 107.1f},
+    {0, 0, 1, 44160, 2048, 384, 1, 31, 127.0f},
     {0, 0, 0, 8192, 8192, 8192, 1, 30, 142.0f},
     {1, 0, 0, 8192, 8192, 8192, 1, 51, 1330.0f},
     {0, 0, 0, 4096, 4096, 4096, 1, 30, 140.6f},
