@@ -51,14 +51,14 @@ __global__ void __launch_bounds__(512) mfma_ceiling_kernel_f64(const uint32_t *s
     }
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// fp16: v_mfma_f32_16x16x32_f16, the instruction of the HGEMM fast path (16 independent accumulators; one operand
+// register repeats for four consecutive MFMAs, as it does in the kernel's walk over its blocks).
+// fp32: v_mfma_f32_32x32x2_f32, the instruction of the SGEMM fast path.
 template <bool F16>
 __global__ void __launch_bounds__(512) mfma_ceiling_kernel(const uint32_t *src, float *out, long long *clk, int iters)
 {
-    f32x16 acc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
     union { uint32_t u[4]; f16x8 h; float f[4]; } a[4], b[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -67,20 +67,41 @@ __global__ void __launch_bounds__(512) mfma_ceiling_kernel(const uint32_t *src, 
             a[q].u[e] = src[(threadIdx.x * 4 + q) * 4 + e];
             b[q].u[e] = src[8192 + (threadIdx.x * 4 + q) * 4 + e];
         }
-    const long long t0 = clock64(), w0 = wall_clock64();
-    for (int it = 0; it < iters; ++it) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if constexpr (F16) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i % 4].h, b[(i / 2) % 4].h, acc[i], 0, 0, 0);
-            else acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i % 4].f[0], b[(i / 2) % 4].f[0], acc[i], 0, 0, 0);
-        }
-    }
-    const long long t1 = clock64(), w1 = wall_clock64();
     float s = 0.0f;
+    long long t0, t1, w0, w1;
+    if constexpr (F16) {
+        f32x4 acc[16];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        t0 = clock64(), w0 = wall_clock64();
+        for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s += acc[i][e];
+            for (int i = 0; i < 16; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i / 4].h, b[i % 4].h, acc[i], 0, 0, 0);
+        }
+        t1 = clock64(), w1 = wall_clock64();
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s += acc[i][e];
+    } else {
+        f32x16 acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][e] = 0.0f;
+        t0 = clock64(), w0 = wall_clock64();
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i % 4].f[0], b[(i / 2) % 4].f[0], acc[i], 0, 0, 0);
+        }
+        t1 = clock64(), w1 = wall_clock64();
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s += acc[i][e];
+    }
     out[blockIdx.x * blockDim.x + threadIdx.x] = s;
     if (threadIdx.x == 0 && blockIdx.x == 0) {
         clk[0] = t1 - t0;
@@ -106,7 +127,7 @@ extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *t
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return MMBO_ERR_NO_DEVICE;
     const int blocks = prop.multiProcessorCount, threads = 512;
-    const int iters = dtype == MMBO_F16 ? 20000 : dtype == MMBO_F32 ? 10000 : 5000;
+    const int iters = dtype == MMBO_F16 ? 100000 : dtype == MMBO_F32 ? 10000 : 5000;      // 15-25 ms per launch: the clock has settled
 
     // operands: 1.0 everywhere, or uniform [-0.3, 0.3) with every mantissa bit in play
     std::vector<uint32_t> h(16384);
@@ -160,8 +181,9 @@ extern "C" int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *t
         }
         long long c[2] = {0, 1};
         if (hipMemcpy(c, d_clk, 16, hipMemcpyDeviceToHost) != hipSuccess || ms <= 0.0f) break;
-        const double flops_per_mfma = dtype == MMBO_F16 ? 32768.0 : dtype == MMBO_F32 ? 4096.0 : 2048.0;
-        *tflops = (double)blocks * (threads / 64) * iters * 8.0 * flops_per_mfma / (ms * 1e-3) * 1e-12;
+        // flop per loop iteration per wavefront: 16 x 16x16x32 (fp16), 8 x 32x32x2 (fp32), 8 x 16x16x4 (fp64)
+        const double flops_per_iter = dtype == MMBO_F16 ? 16 * 16384.0 : dtype == MMBO_F32 ? 8 * 4096.0 : 8 * 2048.0;
+        *tflops = (double)blocks * (threads / 64) * iters * flops_per_iter / (ms * 1e-3) * 1e-12;
         *shader_mhz = c[1] > 0 ? (double)c[0] / (double)c[1] * 100.0 : 0.0;
         rc = MMBO_OK;
     } while (false);

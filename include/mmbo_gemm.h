@@ -118,12 +118,13 @@ int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsi
 int mmbo_release_workspace(void);
 
 /* Measures what the MFMA pipes of the current device sustain with nothing else running: a register-only loop
- * of v_mfma_f32_32x32x16_f16 (MMBO_F16), v_mfma_f32_32x32x2_f32 (MMBO_F32) or v_mfma_f64_16x16x4_f64 (MMBO_F64),
+ * of v_mfma_f32_16x16x32_f16 (MMBO_F16), v_mfma_f32_32x32x2_f32 (MMBO_F32) or v_mfma_f64_16x16x4_f64 (MMBO_F64) -- the
+ * instructions of the three fast paths --,
  * two wavefronts per SIMD, operands
  * all 1.0 (random_operands = 0) or uniform random (1).  Returns TFLOP/s and the average shader clock in MHz.
  * Counterpart of the reference's issue-only probe kernel src/gemm/assembly/error_kernel_000.s and of the
  * hard-coded 6.5 TFLOP/s peak its harness divides by (src/gemm/test.cc:88).  Allocates and frees a few
- * hundred KB; takes a few milliseconds. */
+ * hundred KB; takes some tens of milliseconds. */
 int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *tflops, double *shader_mhz);
 
 const char *mmbo_status_string(int status);
