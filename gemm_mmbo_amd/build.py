@@ -38,8 +38,9 @@ def _units():
         for tile in range(NUM_RING_TILES):
             units.append(("inst_ring.hip", f"inst_ring_{dtype}_{tile}.o",
                           [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
-    for tile in range(NUM_X16_TILES):
-        units.append(("inst_x16.hip", f"inst_x16_{tile}.o", [f"-DMMBO_TILE={tile}"]))
+    for dtype in (0, 1):
+        for tile in range(NUM_X16_TILES):
+            units.append(("inst_x16.hip", f"inst_x16_{dtype}_{tile}.o", [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
     for tile in range(NUM_F64_TILES):
         units.append(("inst_dgemm.hip", f"inst_dgemm_{tile}.o", [f"-DMMBO_TILE={tile}"]))
     extra = os.path.join(CSRC, "extra_units.txt")

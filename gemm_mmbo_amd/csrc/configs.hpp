@@ -63,7 +63,8 @@ constexpr RingRow kRingTiles[NUM_RING_TILES] = {
 };
 constexpr int ring_bk(int dtype) { return dtype == 0 ? 16 : 32; }
 
-// HGEMM tiles of the 16x16x32-MFMA ring kernel with accumulation-register accumulators (hgemm_x16.hpp); depthU 32.
+// Tiles of the 16x16-block ring kernel with accumulation-register accumulators (gemm_x16.hpp), both element types;
+// depthU is 32 (fp16) / 16 (fp32).
 // Config ids continue after the ring and wide ones:  x16_tile + NUM_X16_TILES * split_index.
 constexpr int NUM_X16_TILES = 5;
 constexpr RingRow kX16Tiles[NUM_X16_TILES] = {

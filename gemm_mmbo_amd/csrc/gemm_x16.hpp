@@ -1,6 +1,8 @@
-// HGEMM ring kernel on v_mfma_f32_16x16x32_f16 with the accumulators pinned to the accumulation registers.
+// Ring kernel on 16 x 16 MFMA blocks (v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32) with the accumulators pinned
+// to the accumulation registers.
 //
-// Same structure as gemm_ring.hpp (whole tiles only; K in 32-wide slices through a ring of LDS buffers filled by
+// Same structure as gemm_ring.hpp (whole tiles only; K in slices of 64 bytes per row -- 32 halves or 16 floats --
+// through a ring of LDS buffers filled by
 // global->LDS direct loads; fragments double-buffered in registers; one barrier per slice), and the same recipe
 // as the reference's kernels (src/gemm/ref/Kernels.cpp:412-747).  Two differences, both about energy: MI355X
 // lowers its clock under the power that fp16 MFMAs on real data draw, so what a kernel costs per flop outside
@@ -60,6 +62,21 @@ __device__ __forceinline__ void mfma_acc(const u32x4 &a, const u32x4 &b)
         asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
                      :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63);
 }
+// fp32: acc block BASE/4 += (one k of four per lane group) A x B; called four times per fragment pair
+template <int BASE, int NACC>
+__device__ __forceinline__ void mfma_acc_f32(uint32_t a, uint32_t b)
+{
+    static_assert(BASE % 4 == 0 && BASE + 4 <= NACC, "accumulator block out of range");
+    if constexpr (NACC > 128)
+        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
+    else if constexpr (NACC > 64)
+        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
+    else
+        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
+                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63);
+}
 template <int NACC>
 __device__ __forceinline__ void acc_zero()
 {
@@ -90,20 +107,24 @@ __device__ __forceinline__ float acc_read()
 //     block, four consecutive k-rows x 32 bytes; its blocks sit 8 k-rows apart.  The chunk index is XORed with a
 //     mask of k so that the four k-rows of a block fall into different 64-byte groups and the two blocks served
 //     in one pass into different halves of a group.
-template <bool KC, int R, int NW>
+template <typename T, bool KC, int R, int NW>
 struct Tile {
+    static constexpr int ESZ = sizeof(T);
     static constexpr int BYTES = R * 64;
     static constexpr int INSTRS = R / 16;
     static_assert(INSTRS % NW == 0, "tile must split evenly over the wavefronts");
     static constexpr int LPW = INSTRS / NW;
-    static constexpr int ROW_BYTES = R * 2;
+    static constexpr int ROW_BYTES = R * ESZ;
     static constexpr int CPR = ROW_BYTES / 16;
     static constexpr int KPI = 1024 / ROW_BYTES;
-    static_assert(KC || R == 64 || R == 128 || R == 256, "RC tile: a k-row is 128, 256 or 512 bytes");
+    static_assert(KC || R == 64 || R == 128 || R == 256, "RC tile: a k-row is 128 to 1024 bytes, a power of two");
 
     __device__ static inline uint32_t rc_mask(uint32_t k)
     {
-        if constexpr (ROW_BYTES % 256 == 0) return ((k & 3) << 2) | (((k >> 3) & 1) << 1);
+        // fp32 (ds_read_b32: lane group g = l / 16 reads k-row 4g + t, 16 consecutive rows = 64 bytes): the four
+        // groups of one read go to the four 64-byte quarters of the 256-byte bank span
+        if constexpr (ESZ == 4) return ((k >> 2) & 3) << 2;
+        else if constexpr (ROW_BYTES % 256 == 0) return ((k & 3) << 2) | (((k >> 3) & 1) << 1);
         else return (((k >> 1) & 1) << 2) | (((k >> 3) & 1) << 1);    // 128-byte k-rows alternate between bank halves
     }
     __device__ static inline uint32_t kc_swz(uint32_t row) { return (row >> 1) & 3; }
@@ -117,21 +138,24 @@ struct Tile {
         if constexpr (KC) {
             uint32_t row = q * 16 + (lane >> 2);
             uint32_t chunk = (lane & 3) ^ kc_swz(row);
-            return row * ld * 2 + chunk * 16;
+            return row * ld * ESZ + chunk * 16;
         } else {
             uint32_t k = q * KPI + lane / CPR;
             uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-            return k * ld * 2 + chunk * 16;
+            return k * ld * ESZ + chunk * 16;
         }
     }
 };
 
-// Fragments of one operand of one wavefront for one slice: F blocks of 16 rows x 32 k, four registers each.
-// Lane l holds row l % 16, k = (l / 16) * 8 + 0..7 -- the operand layout of the 16x16x32 MFMA, for both operands.
-template <bool KC, int R, int NW, int F>
+// Fragments of one operand of one wavefront for one slice: F blocks of 16 rows x one slice of k, four registers each.
+// fp16: lane l holds row l % 16, k = (l / 16) * 8 + 0..7 -- the operand layout of the 16x16x32 MFMA.
+// fp32: lane l holds row l % 16, k = (l / 16) * 4 + t in register t -- register t of both operands feeds the t-th of
+// four 16x16x4 MFMAs (whose lane group g then contracts k = 4g + t: any four k do, as long as A and B agree).
+template <typename E, bool KC, int R, int NW, int F>
 struct Frags {
-    using T = Tile<KC, R, NW>;
-    static constexpr int RPF = KC ? 1 : 2;          // LDS reads per fragment
+    using T = Tile<E, KC, R, NW>;
+    static constexpr int ESZ = sizeof(E);
+    static constexpr int RPF = KC ? 1 : (ESZ == 2 ? 2 : 4);          // LDS reads per fragment
     static constexpr int NOPS = F * RPF;
     u32x4 x[F];
 
@@ -142,6 +166,13 @@ struct Frags {
         Addr ad;
         if constexpr (KC) {
             ad.a[0] = T::kc_off(r0 + (lane & 15), lane >> 4);                     // + f*16*64 per block
+        } else if constexpr (ESZ == 4) {
+            const uint32_t r = lane & 15, g = lane >> 4;
+#pragma unroll
+            for (int f = 0; f < F; ++f) {
+                uint32_t m = r0 + f * 16 + r;
+                ad.a[f] = T::rc_off(4 * g, m >> 2) + (m & 3) * 4;                 // + t k-rows: not in the swizzle mask
+            }
         } else {
             // transposing read: lane j of a 16-lane block points at k-row j/4, rows 4*(j%4)..+3, and receives
             // (k-rows 0..3) x (row j); block b covers k = 8b + 4h + 0..3 with its h-th read
@@ -162,6 +193,8 @@ struct Frags {
         constexpr int f = OP / RPF, h = OP % RPF;
         if constexpr (KC) {
             x[f] = lds_read_b128<f * 16 * 64>(tile + ad.a[0]);
+        } else if constexpr (ESZ == 4) {
+            x[f][h] = ring::lds_read_b32<h * T::ROW_BYTES>(tile + ad.a[f]);
         } else {
             u32x2 v = lds_read_tr16_b64<h * 4 * T::ROW_BYTES>(tile + ad.a[f]);
             x[f][2 * h] = v[0];
@@ -176,23 +209,25 @@ struct Frags {
 
 }  // namespace x16
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
 struct X16Cfg {
     static constexpr int NW = WM * WN, NT = NW * 64;
-    static constexpr int BK = 32;
+    static constexpr int ESZ = sizeof(T);
+    static constexpr int BK = 64 / ESZ;                           // one slice: 64 bytes per row
+    static constexpr int MPF = ESZ == 2 ? 1 : 4;                  // MFMAs per fragment pair
     static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 16, FN = TN / 16;
     static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA block");
     static constexpr int NACC = FM * FN * 4 > 128 ? 256 : FM * FN * 4 > 64 ? 128 : 64;    // accumulation registers claimed
     static_assert(FM * FN * 4 <= 256, "wave tile needs more than 256 accumulator registers");
-    using TileA = x16::Tile<TA, BM, NW>;
-    using TileB = x16::Tile<!TB, BN, NW>;
-    using FragA = x16::Frags<TA, BM, NW, FM>;
-    using FragB = x16::Frags<!TB, BN, NW, FN>;
+    using TileA = x16::Tile<T, TA, BM, NW>;
+    using TileB = x16::Tile<T, !TB, BN, NW>;
+    using FragA = x16::Frags<T, TA, BM, NW, FM>;
+    using FragB = x16::Frags<T, !TB, BN, NW, FN>;
     static constexpr int SLICE_BYTES = TileA::BYTES + TileB::BYTES;
     static constexpr int LDS_BYTES = DEPTH * SLICE_BYTES;
     static_assert(LDS_BYTES <= 160 * 1024, "ring does not fit the 160 KB of LDS");
     static constexpr int BATCH = TileA::LPW + TileB::LPW;         // direct loads per thread per slice
-    static constexpr int NMFMA = FM * FN;
+    static constexpr int NMFMA = FM * FN * MPF;
     static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
 };
 
@@ -202,18 +237,18 @@ struct X16Cfg {
 // EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
 // one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0, bool PAIR = (TA || !TB),
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0, bool PAIR = (TA || !TB),
           int EVEN_OP = (TA ? 0 : 1)>
 __global__ void __launch_bounds__(WM * WN * 64)
-hgemm_x16_kernel(const GemmArgs args)
+gemm_x16_kernel(const GemmArgs args)
 {
     using namespace x16;
-    using Cfg = X16Cfg<TA, TB, BM, BN, WM, WN, DEPTH>;
+    using Cfg = X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>;
     using TileA = typename Cfg::TileA;
     using TileB = typename Cfg::TileB;
     using FragA = typename Cfg::FragA;
     using FragB = typename Cfg::FragB;
-    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC, ESZ = Cfg::ESZ, MPF = Cfg::MPF;
 
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -235,12 +270,12 @@ hgemm_x16_kernel(const GemmArgs args)
 
     const char *gA = static_cast<const char *>(args.A) +
                      ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda + k_begin
-                                                          : (int64_t)k_begin * lda + row0)) * 2;
+                                                          : (int64_t)k_begin * lda + row0)) * ESZ;
     const char *gB = static_cast<const char *>(args.B) +
                      ((int64_t)batch * args.strideB + (TB ? (int64_t)k_begin * ldb + col0
-                                                          : (int64_t)col0 * ldb + k_begin)) * 2;
-    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * 2;
-    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * 2;
+                                                          : (int64_t)col0 * ldb + k_begin)) * ESZ;
+    const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * ESZ;
+    const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * ESZ;
 
     uint32_t offA[TileA::LPW], offB[TileB::LPW];
 #pragma unroll
@@ -327,9 +362,14 @@ hgemm_x16_kernel(const GemmArgs args)
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // boustrophedon over the FM x FN blocks: consecutive MFMAs share one operand register, also at the row
-            // ends (a register-only loop of these MFMAs runs 3 % faster when one operand repeats than when both change)
-            constexpr int i = m / FN, j = (i & 1) ? FN - 1 - m % FN : m % FN;
-            if constexpr (!(ABLATE & 4)) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
+            // ends (a register-only loop of these MFMAs runs 3 % faster when one operand repeats than when both change);
+            // fp32 walks the blocks four times, once per k register, so an accumulator recurs every FM*FN MFMAs
+            constexpr int tt = m / (FM * FN), ij = m % (FM * FN);
+            constexpr int i = ij / FN, j = (i & 1) ? FN - 1 - ij % FN : ij % FN;
+            if constexpr (!(ABLATE & 4)) {
+                if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
+                else mfma_acc_f32<(i * FN + j) * 4, NACC>(ca.x[i][tt], cb.x[j][tt]);
+            }
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (!(ABLATE & 2) && m < READ_SPAN) {
                 constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
@@ -536,44 +576,49 @@ hgemm_x16_kernel(const GemmArgs args)
     }
     const float alpha = args.alpha, beta = args.beta;
     const uint32_t ldc = args.ldc;
-    half_t *C = static_cast<half_t *>(args.C) + (int64_t)batch * args.strideC;
+    T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
     const bool vec_c = args.vec_c != 0;
+    typedef typename std::conditional<ESZ == 2, u32x2, u32x4>::type cvec;       // four consecutive rows of one column
     if (vec_c && beta != 0.0f) {
-        // beta != 0 (reference: the fma(C, beta, .) epilogue, MT192x096x08 kernel :3037-3056): all of the wave tile's old C
-        // is requested before the first value is used -- up to 128 registers, free now that the fragments are dead -- so the
-        // read-modify-write runs at memory bandwidth instead of one load latency per block.
-        u32x2 cold[FM * FN];
-        static_for<FM * FN>([&](auto IJ) {
-            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM;
-            cold[decltype(IJ)::value] = *reinterpret_cast<const u32x2 *>(C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16);
-        });
-        static_for<FM * FN>([&](auto IJ) {
-            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
-            half_t *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
-            union { half_t e[4]; u32x2 v2; } io;
-            io.v2 = cold[decltype(IJ)::value];
-            float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
+        // beta != 0 (reference: the fma(C, beta, .) epilogue, MT192x096x08 kernel :3037-3056): a whole column strip of
+        // old C (fp16: the whole wave tile) is requested before its first value is used, so the read-modify-write runs
+        // at memory bandwidth instead of one load latency per block.
+        constexpr int CHUNK = ESZ == 2 ? FM * FN : FM;                          // blocks requested at once
+        static_for<FM * FN / CHUNK>([&](auto CC) {
+            constexpr int c0 = decltype(CC)::value * CHUNK;
+            cvec cold[CHUNK];
+            static_for<CHUNK>([&](auto Q) {
+                constexpr int ij = c0 + decltype(Q)::value, j = ij / FM, i = ij % FM;
+                cold[decltype(Q)::value] = *reinterpret_cast<const cvec *>(C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16);
+            });
+            static_for<CHUNK>([&](auto Q) {
+                constexpr int ij = c0 + decltype(Q)::value, j = ij / FM, i = ij % FM, base = (i * FN + j) * 4;
+                T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
+                union { T e[4]; cvec v; } io;
+                io.v = cold[decltype(Q)::value];
+                float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) io.e[r] = (half_t)__builtin_fmaf(beta, (float)io.e[r], v[r]);
-            *reinterpret_cast<u32x2 *>(p) = io.v2;
+                for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], v[r]);
+                *reinterpret_cast<cvec *>(p) = io.v;
+            });
         });
         return;
     }
     static_for<FM * FN>([&](auto IJ) {
         constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
-        half_t *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
+        T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
         float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
         if (vec_c) {
-            union { half_t e[4]; u32x2 v2; } io;
+            union { T e[4]; cvec v; } io;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) io.e[r] = (half_t)v[r];
-            *reinterpret_cast<u32x2 *>(p) = io.v2;
+            for (int r = 0; r < 4; ++r) io.e[r] = (T)v[r];
+            *reinterpret_cast<cvec *>(p) = io.v;
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 float o = v[r];
                 if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
-                p[r] = (half_t)o;
+                p[r] = (T)o;
             }
         }
     });

@@ -1,22 +1,24 @@
-// Instantiates the 16x16x32-MFMA HGEMM ring kernel for one tile row: compile with -DMMBO_TILE=<row>
+// Instantiates the 16x16-block ring kernel for one (element type, tile row): compile with
+//   -DMMBO_DTYPE=<0|1> -DMMBO_TILE=<row>
 #include "configs.hpp"
-#include "hgemm_x16.hpp"
+#include "gemm_x16.hpp"
 #include "launch.hpp"
 
-#ifndef MMBO_TILE
-#error "MMBO_TILE selects what this translation unit instantiates"
+#ifndef MMBO_DTYPE
+#error "MMBO_DTYPE and MMBO_TILE select what this translation unit instantiates"
 #endif
 
 namespace mmbo {
 
 namespace {
+using ElemT = typename std::conditional<MMBO_DTYPE == 0, float, half_t>::type;
 constexpr RingRow R = kX16Tiles[MMBO_TILE];
 
 template <bool TA, bool TB, int WM, int WN>
 hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
-    using Cfg = X16Cfg<TA, TB, R.bm, R.bn, WM, WN, R.depth>;
-    auto kernel = hgemm_x16_kernel<TA, TB, R.bm, R.bn, WM, WN, R.depth>;
+    using Cfg = X16Cfg<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
+    auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
     static bool attr_set[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -33,10 +35,10 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 }
 }  // namespace
 
-// The operand that needs transposing LDS reads (two per fragment instead of one) gets the fewer fragments:
+// The operand that needs transposing LDS reads (two or four per fragment instead of one) gets the fewer fragments:
 // A needs them under transA = N, B under transB = T, so TT swaps the wave layout.
 template <>
-hipError_t launch_x16<MMBO_TILE>(int transA, int transB, const GemmArgs &args, hipStream_t stream)
+hipError_t launch_x16<MMBO_DTYPE, MMBO_TILE>(int transA, int transB, const GemmArgs &args, hipStream_t stream)
 {
     if (!transA && !transB) return launch_one<false, false, R.wm, R.wn>(args, stream);
     if (!transA && transB) return launch_one<false, true, R.wm, R.wn>(args, stream);

@@ -23,7 +23,7 @@ namespace {
 constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
 constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
 constexpr int kWideConfig = kStagedConfigs + kRingConfigs;      // HGEMM NN/TT 256x256 ring with 64-k units
-constexpr int kX16Base = kWideConfig + 1;                      // HGEMM 16x16x32-MFMA ring, (x16 tile, split) pairs
+constexpr int kX16Base = kWideConfig + 1;                      // ring on 16x16 MFMA blocks, (x16 tile, split) pairs
 constexpr int kX16Configs = NUM_X16_TILES * NUM_SPLITS;
 constexpr int kNumConfigs = kX16Base + kX16Configs;
 
@@ -121,11 +121,11 @@ hipError_t dispatch_ring(int tile, int ta, int tb, const GemmArgs &a, hipStream_
     return hipErrorInvalidValue;
 }
 
-template <int TILE>
+template <int DTYPE, int TILE>
 hipError_t dispatch_x16(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
 {
-    if (tile == TILE) return launch_x16<TILE>(ta, tb, a, s);
-    if constexpr (TILE + 1 < NUM_X16_TILES) return dispatch_x16<TILE + 1>(tile, ta, tb, a, s);
+    if (tile == TILE) return launch_x16<DTYPE, TILE>(ta, tb, a, s);
+    if constexpr (TILE + 1 < NUM_X16_TILES) return dispatch_x16<DTYPE, TILE + 1>(tile, ta, tb, a, s);
     return hipErrorInvalidValue;
 }
 
@@ -294,7 +294,7 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
         const RingRow &r = c.x16 ? kX16Tiles[c.tile] : kRingTiles[c.tile];
         std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d%s", r.bm, r.bn,
                       ring_bk(dtype), r.bm / r.wm, r.bn / r.wn, r.wm * r.wn, c.split, r.depth,
-                      c.x16 ? "_MFMA16x16x32_ACC" : "");
+                      !c.x16 ? "" : dtype == MMBO_F16 ? "_MFMA16x16x32_ACC" : "_MFMA16x16x4_ACC");
         out->macro_tile_m = r.bm;
         out->macro_tile_n = r.bn;
         out->depth_u = ring_bk(dtype);
@@ -356,8 +356,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
     }
     // ring configs: same tile geometry, deeper prefetch, no edge handling.  Where one applies it replaces the
     // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).  For fp16 the ring
-    // kernel on 16x16x32 MFMAs takes its place (faster than both the 32x32x16 ring and the wide-unit kernel on every
-    // shape swept).
+    // kernel on 16x16 MFMA blocks takes its place (faster than both the 32x32x16 ring and the wide-unit kernel on
+    // every shape swept).
     {
         const ConfigRef c = config_ref(best);
         const TileRow &t = tile_row(dtype, c.tile);
@@ -367,7 +367,14 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
             if (r.bm * r.bn > t.bm * t.bn) continue;
             for (int si = 0; si < NUM_SPLITS; ++si)
                 if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k))
-                    return dtype == MMBO_F16 ? x16_config_id(x16_of_ring[rt], si) : ring_config_id(rt, si);
+                {
+                    if (dtype == MMBO_F16) return x16_config_id(x16_of_ring[rt], si);
+                    // fp32: the x16 kernel's 256 x 256 tile (v_mfma_f32_16x16x4_f32, four wavefronts) measures 1.5-2 %
+                    // faster than the ring kernel's at 8192^3 in NN, TN and TT and 0.8 % slower in NT; the smaller
+                    // tiles are equal within noise and stay with the ring kernel
+                    if (rt == 0 && !(transA == 0 && transB == 1)) return x16_config_id(0, si);
+                    return ring_config_id(rt, si);
+                }
         }
     }
     return best;
@@ -458,7 +465,6 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
-    if (cref.x16 && dtype != MMBO_F16) return MMBO_ERR_INVALID_CONFIG;
 
     // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
     {
@@ -509,7 +515,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     hipError_t e;
     if (f64) e = dispatch_dgemm<0>(cref.tile, transA, transB, a, s);
     else if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
-    else if (cref.x16) e = dispatch_x16<0>(cref.tile, transA, transB, a, s);
+    else if (cref.x16) e = dtype == MMBO_F32 ? dispatch_x16<0, 0>(cref.tile, transA, transB, a, s)
+                                        : dispatch_x16<1, 0>(cref.tile, transA, transB, a, s);
     else if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
                                          : dispatch_ring<1, 0>(cref.tile, transA, transB, a, s);
     else e = dtype == MMBO_F32 ? dispatch_tile<0, 0>(cref.tile, transA, transB, a, s)

@@ -20,7 +20,7 @@ constexpr TunedRow kTuned[] = {
     //dtype ta tb m n k batch id TFLOP/s
     {0, 0, 0, 1024, 1024, 1024, 1, 33, 93.0f},
     {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
-    {0, 1, 0, 4096, 4096, 4096, 1, 30, 137.1f},
+    {0, 1, 0, 4096, 4096, 4096, 1, 51, 145.0f},
     {0, 0, 0, 1023, 777, 513, 1, 10, 30.0f},
     {1, 0, 0, 1023, 777, 513, 1, 10, 39.0f},
     {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
@@ -31,7 +31,7 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 2048, 2048, 2048, 1, 31, 121.0f},
     {1, 0, 0, 2048, 2048, 2048, 1, 53, 761.2f},
     {0, 0, 1, 44160, 2048, 384, 1, 31, 127.0f},
-    {0, 0, 0, 8192, 8192, 8192, 1, 30, 142.0f},
+    {0, 0, 0, 8192, 8192, 8192, 1, 51, 145.3f},
     {1, 0, 0, 8192, 8192, 8192, 1, 51, 1330.0f},
     {0, 0, 0, 4096, 4096, 4096, 1, 30, 140.6f},
     {1, 0, 0, 4096, 4096, 4096, 1, 51, 1245.0f},

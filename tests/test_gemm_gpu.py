@@ -92,7 +92,7 @@ def test_every_config_aligned_interior(dtype):
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
         name = G.config_info(dtype, cid)["name"]
-        if dtype == F32 and ("+3U" in name or "MFMA16x16x32" in name):      # fp16-only kernels
+        if dtype == F32 and "+3U" in name:      # an fp16-only kernel
             with pytest.raises(G.MmboError):
                 U.run_gpu(p, cid)
             continue
@@ -103,13 +103,14 @@ def _ring_ids(dtype):
     """Config ids of the generic direct-to-LDS ring kernel (32x32 MFMA blocks)."""
     import gemm_mmbo_amd as G
     names = {c: G.config_info(dtype, c)["name"] for c in range(G.num_configs(dtype))}
-    return [c for c, nm in names.items() if "DTL1" in nm and "+3U" not in nm and "MFMA16x16x32" not in nm]
+    return [c for c, nm in names.items() if "DTL1" in nm and "+3U" not in nm and "_ACC" not in nm]
 
 
-def _x16_ids():
-    """Config ids of the HGEMM ring kernel on 16x16x32 MFMAs with accumulation-register accumulators."""
+def _x16_ids(dtype=F16):
+    """Config ids of the ring kernel on 16x16 MFMA blocks with accumulation-register accumulators."""
     import gemm_mmbo_amd as G
-    return [c for c in range(G.num_configs(F16)) if "MFMA16x16x32" in G.config_info(F16, c)["name"]]
+    mark = "MFMA16x16x32_ACC" if dtype == F16 else "MFMA16x16x4_ACC"
+    return [c for c in range(G.num_configs(dtype)) if mark in G.config_info(dtype, c)["name"]]
 
 
 def _wide_id():
@@ -161,34 +162,37 @@ def test_ring_kernel_every_config_every_transpose(dtype, ta, tb):
     assert ran == 80
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
-def test_x16_kernel_every_config_every_transpose(ta, tb):
-    """The HGEMM ring kernel on v_mfma_f32_16x16x32_f16 with accumulators pinned to the accumulation registers, by
-    explicit config id: every tile (4 and 8 wavefronts, 64 to 256 accumulator registers) and split-K factor, K
-    shorter and longer than the ring, odd slice counts, beta read-modify-write, batches."""
+def test_x16_kernel_every_config_every_transpose(dtype, ta, tb):
+    """The ring kernel on 16x16 MFMA blocks (v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32) with accumulators pinned
+    to the accumulation registers, by explicit config id: every tile (4 and 8 wavefronts, 64 to 256 accumulator
+    registers) and split-K factor, K shorter and longer than the ring, odd slice counts (the paired-load schedule has an
+    even/odd rhythm), beta read-modify-write, batches."""
     import gemm_mmbo_amd as G
-    ids = _x16_ids()
+    ids = _x16_ids(dtype)
     assert len(ids) == 25
+    bk = 16 if dtype == F32 else 32
     ran = 0
     for cid in ids:
-        d = G.config_info(F16, cid)
-        assert d["depth_u"] == 32
+        d = G.config_info(dtype, cid)
+        assert d["depth_u"] == bk
         bm, bn, sp = d["macro_tile_m"], d["macro_tile_n"], d["split_k"]
         for (tm, tn, slices, alpha, beta, batch) in ((1, 1, 1, 1.0, 0.0, 1), (2, 1, 3, 1.5, 0.5, 1), (1, 3, 7, -1.0, 1.0, 2),
-                                                     (3, 2, 33, 1.0, 0.0, 1)):
-            m, n, k = bm * tm, bn * tn, 32 * slices * sp
-            p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=170 + cid + slices, dist="normal",
-                          c_fill="uniform" if beta else "nan")
+                                                     (3, 2, 33, 1.0, 0.0, 1), (1, 1, 6, 1.0, 0.0, 1)):
+            m, n, k = bm * tm, bn * tn, bk * slices * sp
+            p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, batch=batch, seed=170 + cid + slices,
+                          dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
             _run_and_check(p, cid, label=f"{d['name']} {m}x{n}x{k} b{batch}")
             ran += 1
-    assert ran == 100
+    assert ran == 125
 
 
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
-    ragged border of tiles, against the oracle.  Ragged shapes, fp32 and unaligned operands are refused; ld > dim and
-    the automatic pick work."""
+    ragged border of tiles, against the oracle.  Ragged shapes and unaligned operands are refused; ld > dim and the
+    automatic pick work."""
     import gemm_mmbo_amd as G
     ids = _x16_ids()
     for cid in ids[:2]:
@@ -198,7 +202,7 @@ def test_x16_kernel_chip_block_order_and_refusals():
             _run_and_check(p, cid, label=f"chip blocks {m}x{n}x{k}")
     cid = ids[0]
     for (dtype, m, n, k, offs) in ((F16, 255, 256, 128, (0, 0, 0)), (F16, 256, 300, 128, (0, 0, 0)), (F16, 256, 256, 136, (0, 0, 0)),
-                                   (F16, 256, 256, 128, (1, 0, 0)), (F32, 256, 256, 128, (0, 0, 0))):
+                                   (F16, 256, 256, 128, (1, 0, 0)), (F32, 256, 256, 136, (0, 0, 0))):
         p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
         with pytest.raises(G.MmboError) as e:
             U.run_gpu(p, cid, offs)
@@ -207,6 +211,9 @@ def test_x16_kernel_chip_block_order_and_refusals():
     _run_and_check(p, cid, label="x16 ld>dim")
     assert G.select_config(F16, 0, 0, 8192, 8192, 8192) in ids
     assert G.select_config(F16, 0, 1, 2048, 2048, 2048) in ids
+    assert G.select_config(F32, 1, 0, 8192, 8192, 8192) in _x16_ids(F32)
+    p = U.Problem(F32, 0, 0, 4096, 4352, 48, 1.0, 0.0, seed=301, c_fill="nan")
+    _run_and_check(p, _x16_ids(F32)[0], label="fp32 chip blocks")
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)

@@ -27,7 +27,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 
 #        source file            defines
-UNITS = [("inst_x16.hip", ["-DMMBO_TILE=%d" % t]) for t in range(5)] + \
+UNITS = [("inst_x16.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(5)] + \
         [("inst_ring.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(4)] + \
         [("inst_ring_wide.hip", [])]
 
@@ -108,7 +108,7 @@ def test_no_register_is_touched_while_its_lds_read_is_in_flight(asm_files):
             bad = _inflight_violations(body)
             assert not bad, f"{name}: {bad[:3]}"
             checked += 1
-    assert checked >= 4 * (5 + 8) + 2      # four transposes of every tile, both wide kernels
+    assert checked >= 4 * (10 + 8) + 2     # four transposes of every tile, both wide kernels
 
 
 def test_no_scratch_spills(asm_files):
@@ -132,7 +132,8 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
                 used.update(int(a, 0) for a in re.findall(r"\ba\[(\w+)\]", t))
                 # no accumulation register may appear outside the MFMAs, the zeroing and the read-back
                 if re.search(r"\ba\[?\d", t):
-                    assert t.startswith(("v_mfma_f32_16x16x32_f16", "v_accvgpr_write_b32", "v_accvgpr_read_b32")), (name, t)
+                    assert t.startswith(("v_mfma_f32_16x16x32_f16", "v_mfma_f32_16x16x4_f32", "v_accvgpr_write_b32",
+                                         "v_accvgpr_read_b32")), (name, t)
             m = re.search(r"\.amdhsa_kernel " + re.escape(name) + r"\b.*?\.amdhsa_next_free_vgpr (\d+).*?\.amdhsa_accum_offset (\d+)",
                           text, re.S)
             assert m, name
@@ -140,4 +141,4 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
-    assert seen == 20
+    assert seen == 40
