@@ -1,5 +1,6 @@
 """Headline benchmark: GEMM TFLOP/s at 8192^3 on one MI355X, fp16 (value) and fp32 (in "also"); "also" further
-carries the reference's own workload, DGEMM NT 44160 x 2048 x 384 with alpha = -1, beta = 1, and DGEMM at 8192^3.
+carries the two HBM-bound skinny shapes (achieved algorithmic GB/s), the reference's own workload, DGEMM NT
+44160 x 2048 x 384 with alpha = -1, beta = 1, and DGEMM at 8192^3.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
@@ -20,7 +21,7 @@ METRIC = "GEMM TFLOP/s + % of MFMA peak, fp16 & fp32 at 8192^3, 1 MI355X"
 PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}      # MI355X published dense matrix peaks
 # Bytes per launch that crossed the L2 <-> fabric boundary, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
 # this same command (each scaled by the counter's reading for a plain elementwise pass of known size; the
-# summaries with the commands are profiles/hgemm_x16_8192.txt and profiles/sgemm_ring_8192.txt).
+# summaries with the commands are profiles/gemm_x16_f16_8192.txt and profiles/sgemm_ring_8192.txt).
 MEASURED_TRAFFIC_BYTES = {"f16": 1.611e9 + 0.135e9, "f32": 5.501e9 + 0.273e9}
 
 
@@ -129,6 +130,38 @@ def dgemm_legs(G, torch, steps, warmup):
     return out
 
 
+def skinny_legs(G, torch, steps, warmup):
+    """The two HBM-bound shapes of the benchmark set (NN, alpha = 1, beta = 0, U[-1,1] inputs) in both element types:
+    time per GEMM (split-K main kernel + reduction) from events on the launch stream, algorithmic bytes / time against
+    the 8 TB/s HBM peak.  Parity of these shapes at full size is in tests/test_gemm_gpu.py."""
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    out = {}
+    for dname, dtype, tdt, esz in (("fp16", G.F16, torch.float16, 2), ("fp32", G.F32, torch.float32, 4)):
+        for (m, n, k) in ((4096, 128, 4096), (128, 4096, 8192)):
+            A = (torch.rand(m * k, device="cuda", generator=gen) * 2 - 1).to(tdt)
+            B = (torch.rand(k * n, device="cuda", generator=gen) * 2 - 1).to(tdt)
+            C = torch.empty(m * n, device="cuda", dtype=tdt)
+            cid = G.select_config(dtype, 0, 0, m, n, k, 1)
+            for _ in range(warmup):
+                G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
+            e1.record(stream)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / steps * 1e3
+            nbytes = (m * k + k * n + m * n) * esz
+            out[f"{dname}_{m}x{n}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / us * 1e-3, 1),
+                                            "frac_of_hbm_peak": round(nbytes / us * 1e-3 / 8000.0, 4),
+                                            "tflops": round(2.0 * m * n * k / us * 1e-6, 1),
+                                            "tile_config": G.config_info(dtype, cid)["name"]}
+    return out
+
+
 def cpu_baseline(dtype, m, n, k, hA, hB):
     """The oracle's native-precision CPU GEMM (fp16 operands widened to fp32, fp32 multiply-add chains) on
     the same operands, all host cores, whole problem once."""
@@ -182,6 +215,7 @@ def main():
         torch.cuda.empty_cache()
 
     f64 = dgemm_legs(G, torch, args.steps, args.warmup) if args.only in (None, "f64") else {}
+    skinny = skinny_legs(G, torch, args.steps, args.warmup) if not args.only else {}
     if args.only == "f64":
         print(json.dumps({"metric": METRIC, "also": f64}))
         return
@@ -224,6 +258,8 @@ def main():
                        "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
                        "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
                        "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}
+    if skinny:
+        out.setdefault("also", {})["skinny_nn_hbm_bound"] = skinny
     if f64:
         out.setdefault("also", {}).update(f64)
         out["parity_ok"] = bool(out["parity_ok"] and f64["fp64_hpl_max_rel_err"] <= f64["fp64_hpl_rel_err_limit"]
