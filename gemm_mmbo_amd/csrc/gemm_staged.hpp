@@ -9,6 +9,8 @@
 // write), rebuilt around matrix instructions and 64-wide wavefronts.
 #pragma once
 
+#include <type_traits>
+
 #include "gemm_common.hpp"
 
 namespace mmbo {
@@ -328,23 +330,73 @@ gemm_staged_kernel(const GemmArgs args)
 }
 
 // Split-K reduction: C = alpha * sum_s ws[s] + beta * C, splits added in ascending order so the
-// result does not depend on scheduling.  One thread per element of C.
-template <typename T>
+// result does not depend on scheduling.  The workspace is [split][batch][n][m] fp32, dense, so four consecutive
+// rows of one column are one 16-byte load per split; a thread owns such a group when m % 4 == 0 (VEC4), one
+// element otherwise.  All loads of a thread are independent and issued before the first add (the loop over the
+// splits is unrolled for the split factors the library uses); the adds keep the order.
+template <typename T, bool VEC4>
 __global__ void __launch_bounds__(256)
 splitk_reduce_kernel(const GemmArgs args)
 {
+    constexpr int W = VEC4 ? 4 : 1;
     const size_t mn = (size_t)args.m * args.n;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * W;
     const uint32_t batch = blockIdx.z;
     if (idx >= mn) return;
     const uint32_t row = (uint32_t)(idx % args.m), col = (uint32_t)(idx / args.m);
-    float s = 0.0f;
-    for (uint32_t sp = 0; sp < args.splits; ++sp)
-        s += args.ws[((size_t)sp * args.batch + batch) * mn + idx];
+    const size_t stride = (size_t)args.batch * mn;                  // one split further
+    const float *w = args.ws + (size_t)batch * mn + idx;
+    float s[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) s[e] = 0.0f;
+    auto add_splits = [&](auto NS, uint32_t first) {
+        constexpr int ns = decltype(NS)::value;
+        float v[ns][W];
+#pragma unroll
+        for (int q = 0; q < ns; ++q) {
+            const float *p = w + (size_t)(first + q) * stride;
+            if constexpr (VEC4) {
+                f32x4 t = *reinterpret_cast<const f32x4 *>(p);
+                v[q][0] = t[0]; v[q][1] = t[1]; v[q][2] = t[2]; v[q][3] = t[3];
+            } else {
+                v[q][0] = *p;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < ns; ++q)
+#pragma unroll
+            for (int e = 0; e < W; ++e) s[e] += v[q][e];
+    };
+    uint32_t sp = 0;
+    for (; sp + 8 <= args.splits; sp += 8) add_splits(std::integral_constant<int, 8>{}, sp);
+    if (sp + 4 <= args.splits) { add_splits(std::integral_constant<int, 4>{}, sp); sp += 4; }
+    if (sp + 2 <= args.splits) { add_splits(std::integral_constant<int, 2>{}, sp); sp += 2; }
+    if (sp < args.splits) add_splits(std::integral_constant<int, 1>{}, sp);
+
     T *p = static_cast<T *>(args.C) + (int64_t)batch * args.strideC + (size_t)col * args.ldc + row;
-    float o = args.alpha * s;
-    if (args.beta != 0.0f) o = __builtin_fmaf(args.beta, (float)*p, o);
-    *p = (T)o;
+    const float alpha = args.alpha, beta = args.beta;
+    if (VEC4 && args.vec_c) {
+        typedef typename std::conditional<sizeof(T) == 4, u32x4, u32x2>::type cvec;
+        union { T e[4]; cvec v; } io;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = alpha * s[e];
+        if (beta != 0.0f) {
+            io.v = *reinterpret_cast<const cvec *>(p);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = __builtin_fmaf(beta, (float)io.e[e], o[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) io.e[e] = (T)o[e];
+        *reinterpret_cast<cvec *>(p) = io.v;
+    } else {
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            float o = alpha * s[e];
+            if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[e], o);
+            p[e] = (T)o;
+        }
+    }
 }
 
 }  // namespace mmbo

@@ -230,9 +230,15 @@ double model_time_f64(int tile, size_t m, size_t n, size_t k, int batch)
 hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t stream)
 {
     size_t mn = (size_t)args.m * args.n;
-    dim3 grid((unsigned)ceil_div(mn, 256), 1, args.batch);
-    if (dtype == MMBO_F32) hipLaunchKernelGGL(splitk_reduce_kernel<float>, grid, dim3(256), 0, stream, args);
-    else hipLaunchKernelGGL(splitk_reduce_kernel<half_t>, grid, dim3(256), 0, stream, args);
+    const bool vec4 = args.m % 4 == 0;                   // a thread then owns four consecutive rows of one column
+    dim3 grid((unsigned)ceil_div(vec4 ? mn / 4 : mn, 256), 1, args.batch);
+    if (dtype == MMBO_F32) {
+        if (vec4) hipLaunchKernelGGL((splitk_reduce_kernel<float, true>), grid, dim3(256), 0, stream, args);
+        else hipLaunchKernelGGL((splitk_reduce_kernel<float, false>), grid, dim3(256), 0, stream, args);
+    } else {
+        if (vec4) hipLaunchKernelGGL((splitk_reduce_kernel<half_t, true>), grid, dim3(256), 0, stream, args);
+        else hipLaunchKernelGGL((splitk_reduce_kernel<half_t, false>), grid, dim3(256), 0, stream, args);
+    }
     return hipGetLastError();
 }
 
