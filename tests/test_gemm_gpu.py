@@ -209,6 +209,12 @@ def test_x16_kernel_chip_block_order_and_refusals():
         assert e.value.status == 5
     p = U.Problem(F16, 1, 0, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71, dist="normal")
     _run_and_check(p, cid, label="x16 ld>dim")
+    # C needs no alignment: an odd element offset and an odd ldc take the element-wise epilogue, with and without beta
+    for dtype in (F16, F32):
+        for beta in (0.0, 0.5):
+            p = U.Problem(dtype, 0, 1, 256, 512, 192, 1.5, beta, ldc=259, seed=72, dist="normal" if dtype == F16 else "uniform",
+                          c_fill="uniform" if beta else "nan")
+            _run_and_check(p, _x16_ids(dtype)[1], label="x16 unaligned C", offsets=(0, 0, 1))
     assert G.select_config(F16, 0, 0, 8192, 8192, 8192) in ids
     assert G.select_config(F16, 0, 1, 2048, 2048, 2048) in ids
     assert G.select_config(F32, 1, 0, 8192, 8192, 8192) in _x16_ids(F32)
