@@ -1,4 +1,6 @@
 // Instantiates the fp64 kernel for one tile row: compile with -DMMBO_TILE=<row>
+#include <atomic>
+
 #include "configs.hpp"
 #include "dgemm.hpp"
 #include "launch.hpp"
@@ -17,15 +19,15 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
     using Cfg = DgemmCfg<TA, TB, R.bm, R.bn, R.bk, R.wm, R.wn>;
     auto kernel = dgemm_kernel<TA, TB, R.bm, R.bn, R.bk, R.wm, R.wn>;
-    static bool attr_set[64] = {};
+    static std::atomic<bool> attr_set[64];           // zero-initialised; several host threads may race to set it: harmless
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
+    if (dev >= 0 && dev < 64 && !attr_set[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
         if (e != hipSuccess) return e;
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     dim3 grid(args.nwg0 * args.nwg1, 1, args.batch);
     hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);

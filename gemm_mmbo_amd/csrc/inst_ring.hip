@@ -1,5 +1,7 @@
 // Instantiates the ring kernel for one (element type, ring tile row): compile with
 //   -DMMBO_DTYPE=<0|1> -DMMBO_TILE=<row>
+#include <atomic>
+
 #include "configs.hpp"
 #include "gemm_ring.hpp"
 #include "launch.hpp"
@@ -19,15 +21,15 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
     using Cfg = RingCfg<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
     auto kernel = gemm_ring_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
-    static bool attr_set[64] = {};
+    static std::atomic<bool> attr_set[64];           // zero-initialised; several host threads may race to set it: harmless
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
+    if (dev >= 0 && dev < 64 && !attr_set[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 Cfg::LDS_BYTES);
         if (e != hipSuccess) return e;
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     dim3 grid(args.nwg0 * args.nwg1, 1, args.batch * args.splits);
     hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
