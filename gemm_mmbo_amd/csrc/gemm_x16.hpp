@@ -231,8 +231,9 @@ struct X16Cfg {
     static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
 };
 
-// ABLATE: timing probe as in gemm_ring.hpp (bit 0 no direct loads, bit 1 no LDS reads, bit 2 no MFMAs); results
-// are wrong by design and the library only instantiates ABLATE = 0.
+// ABLATE: timing probe as in gemm_ring.hpp (bit 0 no direct loads, bit 1 no LDS reads, bit 2 no MFMAs: results are
+// wrong by design; bit 3 writes each work-group's start, loop start, loop end and end times (100 MHz counter) to
+// args.ws[4 * work-group ..]).  The library only instantiates ABLATE = 0.
 // PAIR: fetch two slices of one operand per iteration (see mfma_and_read); on when an operand is k-contiguous.
 // EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
@@ -256,6 +257,8 @@ gemm_x16_kernel(const GemmArgs args)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
+    long long t_probe[4] = {0, 0, 0, 0};
+    if constexpr ((ABLATE & 8) != 0) t_probe[0] = wall_clock64();
 
     uint32_t wg0, wg1;
     if (args.chip_block) chip_block_remap(blockIdx.x, args.nwg0, args.nwg1, wg0, wg1);
@@ -430,6 +433,7 @@ gemm_x16_kernel(const GemmArgs args)
     // that may stay in flight.
     int buf = 0;                                                     // s % DEPTH
     int s = 0;
+    if constexpr ((ABLATE & 8) != 0) t_probe[1] = wall_clock64();
     if constexpr (!PAIR) {
 #pragma unroll
         for (int q = 0; q < DEPTH; ++q)
@@ -554,6 +558,7 @@ gemm_x16_kernel(const GemmArgs args)
 #undef MMBO_WAIT_VM
 #undef MMBO_WAIT_LGKM0
 
+    if constexpr ((ABLATE & 8) != 0) t_probe[2] = wall_clock64();
     // the last MFMAs' results must have landed before they are read back
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
@@ -604,24 +609,61 @@ gemm_x16_kernel(const GemmArgs args)
         });
         return;
     }
-    static_for<FM * FN>([&](auto IJ) {
-        constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
-        T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
-        float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
-        if (vec_c) {
+    // beta == 0: C is never read.  The aligned and the element-wise variant are separate straight-line sequences: with
+    // the choice made per block the epilogue was bound by instruction issue (64 blocks x ~20 instructions with two
+    // branches each took 7 us of a 220 us tile at 8192^3, whatever the number of work-groups writing at the time).
+    if (vec_c && ESZ == 2 && FM % 2 == 0) {
+        // fp16: a lane's four rows are 8 bytes, a column of one block 32 bytes -- a quarter of a cache line per write
+        // request.  Two vertically adjacent blocks are stored together: v_permlane16_swap hands the lanes of the even
+        // 16-lane rows their lower neighbour's four rows of the upper block and the odd rows their upper neighbour's
+        // of the lower block, so every lane stores 16 contiguous bytes and a column gets 64 per instruction.
+        const uint32_t q = lane >> 4;
+        const uint32_t prow0 = row0 + wm * Cfg::TM + ((q & 1) ? 4 * q + 12 : 4 * q);
+        static_for<FM * FN / 2>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
+            constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
+            union { T e[4]; uint32_t u[2]; } x, y;
+            x.e[0] = (T)(alpha * acc_read<b0>());     x.e[1] = (T)(alpha * acc_read<b0 + 1>());
+            x.e[2] = (T)(alpha * acc_read<b0 + 2>()); x.e[3] = (T)(alpha * acc_read<b0 + 3>());
+            y.e[0] = (T)(alpha * acc_read<b1>());     y.e[1] = (T)(alpha * acc_read<b1 + 1>());
+            y.e[2] = (T)(alpha * acc_read<b1 + 2>()); y.e[3] = (T)(alpha * acc_read<b1 + 3>());
+            auto s0 = __builtin_amdgcn_permlane16_swap(x.u[0], y.u[0], false, false);
+            auto s1 = __builtin_amdgcn_permlane16_swap(x.u[1], y.u[1], false, false);
+            T *p = C + (size_t)(wcol0 + j * 16) * ldc + prow0 + i * 16;
+            *reinterpret_cast<u32x4 *>(p) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
+        });
+    } else if (vec_c) {
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
+            T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
             union { T e[4]; cvec v; } io;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) io.e[r] = (T)v[r];
+            io.e[0] = (T)(alpha * acc_read<base>());
+            io.e[1] = (T)(alpha * acc_read<base + 1>());
+            io.e[2] = (T)(alpha * acc_read<base + 2>());
+            io.e[3] = (T)(alpha * acc_read<base + 3>());
             *reinterpret_cast<cvec *>(p) = io.v;
-        } else {
+        });
+    } else {
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
+            T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
+            float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 float o = v[r];
                 if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
                 p[r] = (T)o;
             }
+        });
+    }
+    if constexpr ((ABLATE & 8) != 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        t_probe[3] = wall_clock64();
+        if (tid == 0) {
+            long long *o = reinterpret_cast<long long *>(args.ws) + 4 * (size_t)blockIdx.x;
+            o[0] = t_probe[0]; o[1] = t_probe[1]; o[2] = t_probe[2]; o[3] = t_probe[3];
         }
-    });
+    }
 }
 
 }  // namespace mmbo
