@@ -260,9 +260,16 @@ gemm_x16_kernel(const GemmArgs args)
     long long t_probe[4] = {0, 0, 0, 0};
     if constexpr ((ABLATE & 8) != 0) t_probe[0] = wall_clock64();
 
+    // A work-group walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...: the host launches one work-group per tile,
+    // or, for the 256 x 256 tiles on grids larger than the chip, one per CU (persistent).  Staying resident saves the
+    // dispatch of a new work-group per tile, and the next tile's first loads are in flight while the stores of the
+    // last one are still being acknowledged.  Those stores are older than the loads, and the count-based waits below
+    // only ever wait for more when something older is still outstanding.
+    const uint32_t n_tiles = args.nwg0 * args.nwg1;
+    for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     uint32_t wg0, wg1;
-    if (args.chip_block) chip_block_remap(blockIdx.x, args.nwg0, args.nwg1, wg0, wg1);
-    else wg_remap(blockIdx.x, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
+    if (args.chip_block) chip_block_remap(tile, args.nwg0, args.nwg1, wg0, wg1);
+    else wg_remap(tile, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
     const uint32_t zb = blockIdx.z;
     const uint32_t split = zb / args.batch, batch = zb % args.batch;
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
@@ -577,7 +584,7 @@ gemm_x16_kernel(const GemmArgs args)
             float *p = ws + (size_t)(wcol0 + j * 16) * args.m + wrow0 + i * 16;
             *reinterpret_cast<f32x4 *>(p) = f32x4{acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
         });
-        return;
+        continue;
     }
     const float alpha = args.alpha, beta = args.beta;
     const uint32_t ldc = args.ldc;
@@ -607,7 +614,7 @@ gemm_x16_kernel(const GemmArgs args)
                 *reinterpret_cast<cvec *>(p) = io.v;
             });
         });
-        return;
+        continue;
     }
     // beta == 0: C is never read.  The aligned and the element-wise variant are separate straight-line sequences: with
     // the choice made per block the epilogue was bound by instruction issue (64 blocks x ~20 instructions with two
@@ -660,10 +667,12 @@ gemm_x16_kernel(const GemmArgs args)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         t_probe[3] = wall_clock64();
         if (tid == 0) {
-            long long *o = reinterpret_cast<long long *>(args.ws) + 4 * (size_t)blockIdx.x;
+            long long *o = reinterpret_cast<long long *>(args.ws) + 4 * (size_t)tile;
             o[0] = t_probe[0]; o[1] = t_probe[1]; o[2] = t_probe[2]; o[3] = t_probe[3];
         }
+        t_probe[0] = t_probe[3];
     }
+    }   // tiles of this work-group
 }
 
 }  // namespace mmbo

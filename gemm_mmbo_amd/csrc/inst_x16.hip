@@ -31,7 +31,22 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
         if (e != hipSuccess) return e;
         attr_set[dev].store(true, std::memory_order_release);
     }
-    dim3 grid(args.nwg0 * args.nwg1, 1, args.batch * args.splits);
+    // 256 x 256 tiles (one work-group per CU fits): on grids with more tiles than CUs the work-groups stay resident and
+    // walk the tiles themselves
+    unsigned gx = args.nwg0 * args.nwg1;
+    if (R.bm == 256 && R.bn == 256) {
+        static std::atomic<int> cus[64];
+        int n = dev >= 0 && dev < 64 ? cus[dev].load(std::memory_order_acquire) : 0;
+        if (n == 0) {
+            hipDeviceProp_t prop;
+            e = hipGetDeviceProperties(&prop, dev);
+            if (e != hipSuccess) return e;
+            n = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 1;
+            if (dev >= 0 && dev < 64) cus[dev].store(n, std::memory_order_release);
+        }
+        if (gx > (unsigned)n) gx = (unsigned)n;
+    }
+    dim3 grid(gx, 1, args.batch * args.splits);
     hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
     return hipGetLastError();
 }
