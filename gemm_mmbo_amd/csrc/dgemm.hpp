@@ -8,20 +8,26 @@
 //
 // Register layout of v_mfma_f64_16x16x4_f64 (checked on the device): operand lane l supplies row (column)
 // l%16 at k = l/16; result element e of lane l is D[4*e + l/16][l%16].  A lane's four results are therefore
-// four rows 4 apart.  The A fragment is read with its 16 rows permuted, MFMA row r <- tile row 4*(r%4) + r/4,
-// which turns them into the four CONSECUTIVE rows 4*(l/16) .. +3 of column l%16: 32 contiguous bytes per lane,
-// a full 128-byte line per column across the four lane groups.
+// four rows 4 apart.  The A fragment is read with its 16 rows permuted, MFMA row 4*e + g <- tile row
+// 8*(e/2) + 2*g + e%2 (dgemm_row_of), so that lane group g = l/16 holds rows 2g, 2g+1 (e = 0, 1) and 8+2g, 9+2g
+// (e = 2, 3) of column l%16: a 128-bit access per pair, and the four lane groups of a column together cover 64
+// contiguous bytes per instruction.  (With four consecutive rows per lane instead, an instruction touches 16-byte
+// pieces 32 bytes apart; the C update of a tile then takes about twice as long: the store path of a CU is bound by
+// the number of pieces.)
 #pragma once
 
 #include "gemm_staged.hpp"
 
 namespace mmbo {
 
+// tile row (within a 16-row block) that MFMA row r = 4*e + g of the A operand carries
+__host__ __device__ constexpr int dgemm_row_of(int r) { return 8 * (r >> 3) + 2 * (r & 3) + ((r >> 2) & 1); }
+
 template <bool KC, int LDS_LD>
 __device__ inline uint32_t dfrag_lane_off(int lane, int row0, bool permute_rows)
 {
     int r = lane & 15, g = lane >> 4;
-    if (permute_rows) r = 4 * (r & 3) + (r >> 2);
+    if (permute_rows) r = dgemm_row_of(r);
     if (KC) return (uint32_t)((row0 + r) * LDS_LD + g) * 8;
     return (uint32_t)(g * LDS_LD + row0 + r) * 8;
 }
@@ -48,7 +54,7 @@ struct DgemmCfg {
 };
 
 // C = alpha*acc + beta*C for one wavefront's FM x FN blocks; acc[i][j][e] is
-// C(wrow0 + 16*i + 4*(lane/16) + e, wcol0 + 16*j + lane%16).  beta == 0 never reads C
+// C(wrow0 + 16*i + 8*(e/2) + 2*(lane/16) + e%2, wcol0 + 16*j + lane%16).  beta == 0 never reads C
 // (src/gemm/ref/Kernels.cpp:87); alpha*acc first, then fma(beta, C, .), as the reference's epilogue.
 template <int FM, int FN>
 __device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmArgs &args, uint32_t wrow0,
@@ -59,41 +65,80 @@ __device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmAr
     const int g = lane >> 4, cl = lane & 15;
     double *C = static_cast<double *>(args.C) + (int64_t)batch * args.strideC;
     const bool vec_c = args.vec_c != 0;
+    if (vec_c && wrow0 + FM * 16 <= m && wcol0 + FN * 16 <= n) {
+        // Whole wave tile in range.  The compiler may not move a load of C above an earlier store to C, so a
+        // block-by-block update pays one full memory latency per block; here the old values of HB blocks are
+        // requested together before the first of them is needed.
+        double *p0 = C + (size_t)(wcol0 + cl) * ldc + wrow0 + 2 * g;
+        constexpr int NB = FM * FN, HB = NB < 4 ? NB : 4;
+        static_assert(NB % HB == 0, "blocks per wave tile");
+        if (beta != 0.0) {
+#pragma unroll
+            for (int b0 = 0; b0 < NB; b0 += HB) {
+                f64x2 c[HB][2];
+#pragma unroll
+                for (int b = 0; b < HB; ++b) {
+                    const double *p = p0 + (size_t)((b0 + b) / FM) * 16 * ldc + ((b0 + b) % FM) * 16;
+                    c[b][0] = *reinterpret_cast<const f64x2 *>(p);
+                    c[b][1] = *reinterpret_cast<const f64x2 *>(p + 8);
+                }
+#pragma unroll
+                for (int b = 0; b < HB; ++b) {
+                    const f64x4 &a = acc[(b0 + b) % FM][(b0 + b) / FM];
+                    double *p = p0 + (size_t)((b0 + b) / FM) * 16 * ldc + ((b0 + b) % FM) * 16;
+                    *reinterpret_cast<f64x2 *>(p) = f64x2{__builtin_fma(beta, c[b][0][0], alpha * a[0]),
+                                                          __builtin_fma(beta, c[b][0][1], alpha * a[1])};
+                    *reinterpret_cast<f64x2 *>(p + 8) = f64x2{__builtin_fma(beta, c[b][1][0], alpha * a[2]),
+                                                              __builtin_fma(beta, c[b][1][1], alpha * a[3])};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const f64x4 &a = acc[b % FM][b / FM];
+                double *p = p0 + (size_t)(b / FM) * 16 * ldc + (b % FM) * 16;
+                *reinterpret_cast<f64x2 *>(p) = f64x2{alpha * a[0], alpha * a[1]};
+                *reinterpret_cast<f64x2 *>(p + 8) = f64x2{alpha * a[2], alpha * a[3]};
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
             uint32_t col = wcol0 + j * 16 + cl;
-            uint32_t row = wrow0 + i * 16 + 4 * g;
-            if (col >= n || row >= m) continue;
-            double *p = C + (size_t)col * ldc + row;
-            double v[4];
+            if (col >= n) continue;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = alpha * acc[i][j][e];
-            if (vec_c && row + 4 <= m) {
-                if (beta != 0.0) {
-                    f64x2 c0 = *reinterpret_cast<const f64x2 *>(p), c1 = *reinterpret_cast<const f64x2 *>(p + 2);
-                    v[0] = __builtin_fma(beta, c0[0], v[0]);
-                    v[1] = __builtin_fma(beta, c0[1], v[1]);
-                    v[2] = __builtin_fma(beta, c1[0], v[2]);
-                    v[3] = __builtin_fma(beta, c1[1], v[3]);
-                }
-                *reinterpret_cast<f64x2 *>(p) = f64x2{v[0], v[1]};
-                *reinterpret_cast<f64x2 *>(p + 2) = f64x2{v[2], v[3]};
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (row + e < m) {
-                        double o = v[e];
-                        if (beta != 0.0) o = __builtin_fma(beta, p[e], o);
-                        p[e] = o;
+            for (int h = 0; h < 2; ++h) {       // rows 2g, 2g+1 (h = 0) and 8+2g, 9+2g (h = 1) of the block
+                uint32_t row = wrow0 + i * 16 + 8 * h + 2 * g;
+                if (row >= m) continue;
+                double *p = C + (size_t)col * ldc + row;
+                double v0 = alpha * acc[i][j][2 * h], v1 = alpha * acc[i][j][2 * h + 1];
+                if (vec_c && row + 2 <= m) {
+                    if (beta != 0.0) {
+                        f64x2 c = *reinterpret_cast<const f64x2 *>(p);
+                        v0 = __builtin_fma(beta, c[0], v0);
+                        v1 = __builtin_fma(beta, c[1], v1);
                     }
+                    *reinterpret_cast<f64x2 *>(p) = f64x2{v0, v1};
+                } else {
+                    if (beta != 0.0) v0 = __builtin_fma(beta, p[0], v0);
+                    p[0] = v0;
+                    if (row + 1 < m) {
+                        if (beta != 0.0) v1 = __builtin_fma(beta, p[1], v1);
+                        p[1] = v1;
+                    }
+                }
             }
         }
 }
 
 template <bool TA, bool TB, int BM, int BN, int BK, int WM, int WN>
-__global__ void __launch_bounds__(WM * WN * 64, 2)      // two wavefronts per SIMD: at most 256 registers per lane
+// Eight wavefronts with wave tiles of at most eight blocks (64 accumulator registers, two loader chunks per
+// operand) are held to 128 registers per lane so that two work-groups share a CU (the second argument is
+// wavefronts per SIMD); the others get 256.
+__global__ void __launch_bounds__(WM * WN * 64, (WM * WN >= 8 && (BM / WM / 16) * (BN / WN / 16) <= 8) ? 4 : 2)
 dgemm_kernel(const GemmArgs args)
 {
     using Cfg = DgemmCfg<TA, TB, BM, BN, BK, WM, WN>;
