@@ -1,0 +1,104 @@
+"""Offline tuner: time every tile config on a list of shapes and print rows for csrc/tuned_table.hpp.
+
+The reference keeps an exact-size table for its Tensile kernels, size -> (solution index, measured GFLOP/s)
+(src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:929-1177), and finds the fastest kernel for a size by running all of
+them (src/gemm/benchmark.cc:89-109).  This does the same over this library's config ids, through the C ABI, on the
+GPU it runs on:
+
+    python -m gemm_mmbo_amd.tune                      # the built-in shape list (benchmark configs + HPL sweep points)
+    python -m gemm_mmbo_amd.tune shapes.txt           # one shape per line:  dtype ta tb m n k batch alpha beta
+                                                      # (dtype 0 fp32, 1 fp16, 2 fp64; ta/tb 0 = N, 1 = T)
+
+For every shape it prints the ranking and one line in the table's syntax; paste the lines into kTuned[] and rebuild.
+Configs that do not apply to a shape (whole-tile kernels on ragged shapes) are skipped, as the C ABI refuses them.
+"""
+import sys
+
+BUILTIN = [
+    # dtype ta tb m n k batch alpha beta
+    (0, 0, 0, 1024, 1024, 1024, 1, 1.0, 0.0),
+    (0, 0, 1, 4096, 4096, 4096, 1, 1.5, 0.5), (0, 1, 0, 4096, 4096, 4096, 1, 1.5, 0.5),
+    (0, 0, 0, 1023, 777, 513, 1, 1.0, 0.0), (1, 0, 0, 1023, 777, 513, 1, 1.0, 0.0),
+    (0, 0, 0, 4096, 128, 4096, 1, 1.0, 0.0), (1, 0, 0, 4096, 128, 4096, 1, 1.0, 0.0),
+    (0, 0, 0, 128, 4096, 8192, 1, 1.0, 0.0), (1, 0, 0, 128, 4096, 8192, 1, 1.0, 0.0),
+    (1, 1, 0, 512, 512, 512, 64, 1.0, 1.0),
+    (0, 0, 0, 2048, 2048, 2048, 1, 1.0, 0.0), (1, 0, 0, 2048, 2048, 2048, 1, 1.0, 0.0),
+    (0, 0, 0, 4096, 4096, 4096, 1, 1.0, 0.0), (1, 0, 0, 4096, 4096, 4096, 1, 1.0, 0.0),
+    (0, 0, 0, 8192, 8192, 8192, 1, 1.0, 0.0), (1, 0, 0, 8192, 8192, 8192, 1, 1.0, 0.0),
+    (0, 0, 1, 44160, 2048, 384, 1, -1.0, 1.0), (2, 0, 1, 44160, 2048, 384, 1, -1.0, 1.0),
+    (2, 0, 0, 8192, 8192, 8192, 1, 1.0, 0.0),
+]
+
+
+def time_config(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, cfg, reps):
+    """Milliseconds per launch of one config, or None when the config does not apply to the shape."""
+    tdt = {G.F32: torch.float32, G.F16: torch.float16, G.F64: torch.float64}[dtype]
+    A = (torch.rand(m * k * batch, device="cuda") - 0.5).to(tdt)
+    B = (torch.rand(k * n * batch, device="cuda") - 0.5).to(tdt)
+    C = torch.zeros(m * n * batch, device="cuda", dtype=tdt)
+    lda, ldb = (k if ta else m), (n if tb else k)
+    stream = torch.cuda.current_stream()
+
+    def run():
+        G.gemm_strided_batched(dtype, ta, tb, m, n, k, alpha, A, lda, m * k, B, ldb, k * n, beta, C, m, m * n, batch,
+                               cfg, stream)
+    try:
+        for _ in range(2):
+            run()
+    except G.MmboError:
+        return None
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        run()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def tune(shapes, out=sys.stdout):
+    import torch
+
+    import gemm_mmbo_amd as G
+    if not torch.cuda.is_available():
+        raise RuntimeError("the tuner times kernels: it needs the GPU")
+    rows = []
+    for (dtype, ta, tb, m, n, k, batch, alpha, beta) in shapes:
+        flops = 2.0 * m * n * k * batch
+        reps = 3 if flops > 1e11 else 20
+        res = []
+        for cfg in range(G.num_configs(dtype)):
+            d = G.config_info(dtype, cfg)
+            # split-K and small tiles on the largest problems only cost sweep time
+            if flops > 5e11 and (d["split_k"] > 1 or d["macro_tile_m"] * d["macro_tile_n"] < 128 * 128):
+                continue
+            t = time_config(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, cfg, reps)
+            if t is not None:
+                res.append((t, cfg))
+        res.sort()
+        pick = G.select_config(dtype, ta, tb, m, n, k, batch)
+        t_pick = next((t for t, c in res if c == pick), None)
+        best_t, best = res[0]
+        row = f"    {{{dtype}, {ta}, {tb}, {m}, {n}, {k}, {batch}, {best}, {flops / best_t * 1e-9:.1f}f}},"
+        rows.append(row)
+        print(f"# dtype {dtype} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} batch {batch}: current pick {pick} "
+              f"({'%.1f us' % (t_pick * 1e3) if t_pick else 'not timed'}); fastest: "
+              + "  ".join(f"{c} {G.config_info(dtype, c)['name']} {t * 1e3:.1f} us" for t, c in res[:4]), file=out)
+        print(row, file=out, flush=True)
+    return rows
+
+
+def main(argv):
+    shapes = BUILTIN
+    if len(argv) > 1:
+        shapes = []
+        for line in open(argv[1]):
+            f = line.split("#")[0].split()
+            if f:
+                shapes.append(tuple(int(x) for x in f[:7]) + (float(f[7]), float(f[8])))
+    tune(shapes)
+
+
+if __name__ == "__main__":
+    main(sys.argv)

@@ -198,3 +198,12 @@ def test_python_front_ends_keep_reference_argument_order():
     want = ["m", "n", "k", "alpha", "A", "lda", "B", "ldb", "beta", "C", "ldc", "kernelId"]
     for f in (G.naive_dgemm, G.dgemm_NT, G.naive_sgemm, G.naive_hgemm, G.sgemm_NT, G.sgemm_TN, G.hgemm_NN, G.hgemm_TT):
         assert list(inspect.signature(f).parameters) == want
+
+
+def test_tuner_shape_list_is_valid_and_rows_parse():
+    """Every shape of the offline tuner's built-in list is one the library accepts, and its picks are valid ids."""
+    from gemm_mmbo_amd import tune
+    for (dtype, ta, tb, m, n, k, batch, alpha, beta) in tune.BUILTIN:
+        cid = G.select_config(dtype, ta, tb, m, n, k, batch)
+        assert 0 <= cid < G.num_configs(dtype)
+    # (the timing part needs the GPU: tests/test_gemm_gpu.py)

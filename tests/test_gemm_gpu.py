@@ -429,3 +429,20 @@ def test_mfma_ceiling_probe_reports_plausible_numbers():
     assert 50 < ones32 < 165
     for mhz in (mhz1, mhz2, mhz3):
         assert 500 < mhz < 2600
+
+
+def test_offline_tuner_emits_table_rows_for_small_shapes():
+    """gemm_mmbo_amd/tune.py times every config id and prints rows in tuned_table.hpp's syntax."""
+    import io
+    import re
+
+    import gemm_mmbo_amd as G
+    from gemm_mmbo_amd import tune
+    out = io.StringIO()
+    shapes = [(0, 0, 1, 256, 256, 128, 1, -1.0, 1.0), (1, 1, 0, 300, 200, 96, 2, 1.0, 0.0), (2, 0, 1, 256, 128, 64, 1, -1.0, 1.0)]
+    rows = tune.tune(shapes, out)
+    assert len(rows) == 3
+    for row, s in zip(rows, shapes):
+        m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), ([\d.]+)f\},", row)
+        assert m and tuple(int(x) for x in m.groups()[:7]) == s[:7]
+        assert 0 <= int(m.group(8)) < G.num_configs(s[0]) and float(m.group(9)) > 0
