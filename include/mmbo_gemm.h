@@ -19,7 +19,9 @@
  *     one round-to-nearest-even to binary16 on the store.
  *     MMBO_F64: double A, B, C, alpha, beta (the reference's own element type); fp64 MFMA accumulate;
  *   - the launch is asynchronous on `stream` (a hipStream_t, NULL = the null stream the
- *     reference uses, src/gemm/common.h:12); the caller synchronises;
+ *     reference uses, src/gemm/common.h:12); the caller synchronises.  Configs with GlobalSplitU > 1 keep their
+ *     partial sums in one workspace per device: two such GEMMs must not be in flight on different streams of
+ *     one device at the same time (the same stream, or configs without split-K, are fine);
  *   - config_id selects a row of the tile-config table, like the reference's kernelId
  *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick;
  *   - errors come back as status codes; nothing calls exit() (the reference's HIP_CHECK
