@@ -24,16 +24,16 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 1023, 777, 513, 1, 10, 30.0f},
     {1, 0, 0, 1023, 777, 513, 1, 10, 39.0f},
     {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
-    {1, 0, 0, 4096, 128, 4096, 1, 64, 257.7f},
-    {0, 0, 0, 128, 4096, 8192, 1, 47, 100.1f},
+    {1, 0, 0, 4096, 128, 4096, 1, 37, 272.2f},
+    {0, 0, 0, 128, 4096, 8192, 1, 45, 108.8f},
     {1, 0, 0, 128, 4096, 8192, 1, 64, 398.7f},
     {1, 1, 0, 512, 512, 512, 64, 52, 452.0f},
-    {0, 0, 0, 2048, 2048, 2048, 1, 31, 121.0f},
+    {0, 0, 0, 2048, 2048, 2048, 1, 33, 117.5f},
     {1, 0, 0, 2048, 2048, 2048, 1, 53, 761.2f},
-    {0, 0, 1, 44160, 2048, 384, 1, 31, 127.0f},
+    {0, 0, 1, 44160, 2048, 384, 1, 53, 120.5f},
     {0, 0, 0, 8192, 8192, 8192, 1, 51, 145.3f},
     {1, 0, 0, 8192, 8192, 8192, 1, 51, 1330.0f},
-    {0, 0, 0, 4096, 4096, 4096, 1, 30, 140.6f},
+    {0, 0, 0, 4096, 4096, 4096, 1, 51, 143.6f},
     {1, 0, 0, 4096, 4096, 4096, 1, 51, 1245.0f},
     {2, 0, 1, 44160, 2048, 384, 1, 4, 58.2f},      // the reference's HPL trailing update (src/gemm/run.sh:2-5)
     {2, 0, 0, 8192, 8192, 8192, 1, 0, 69.7f},
