@@ -326,6 +326,41 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
     return MMBO_OK;
 }
 
+// Macro tile (and depthU) of a config id.
+static TileRow config_tile(int dtype, int id)
+{
+    if (dtype == MMBO_F64) return kTilesF64[id];
+    const ConfigRef c = config_ref(id);
+    if (!c.ring) return tile_row(dtype, c.tile);
+    const RingRow &rr = c.x16 ? kX16Tiles[c.tile] : kRingTiles[c.tile];
+    return TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0};
+}
+
+// Per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB.
+static bool tile_span_ok(const TileRow &r, int transA, int transB, size_t lda, size_t ldb, size_t esz)
+{
+    size_t span_a = (transA ? (size_t)r.bm : (size_t)r.bk) * lda * esz;
+    size_t span_b = (transB ? (size_t)r.bk : (size_t)r.bn) * ldb * esz;
+    return span_a < 0x7FFFFF00ull && span_b < 0x7FFFFF00ull;
+}
+
+// The cost model's pick among the staged configs (fp32/fp16), which take any shape and any alignment.
+static int select_staged(int dtype, size_t m, size_t n, size_t k, int batch)
+{
+    int best = 0;
+    double best_t = 0.0;
+    for (int si = 0; si < NUM_SPLITS; ++si) {
+        int split = kSplits[si];
+        for (int tile = 0; tile < NUM_TILES; ++tile) {
+            const TileRow &r = tile_row(dtype, tile);
+            if (split > 1 && ceil_div(k, (size_t)split) < (size_t)2 * r.bk) continue;   // slices too thin
+            double t = model_time(dtype, tile, split, m, n, k ? k : 1, batch);
+            if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
+        }
+    }
+    return best;
+}
+
 int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch)
 {
     if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
@@ -349,17 +384,7 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
             t.batch == batch)
             return t.config_id;
-    int best = 0;
-    double best_t = 0.0;
-    for (int si = 0; si < NUM_SPLITS; ++si) {
-        int split = kSplits[si];
-        for (int tile = 0; tile < NUM_TILES; ++tile) {
-            const TileRow &r = tile_row(dtype, tile);
-            if (split > 1 && ceil_div(k, (size_t)split) < (size_t)2 * r.bk) continue;   // slices too thin
-            double t = model_time(dtype, tile, split, m, n, k ? k : 1, batch);
-            if (best_t == 0.0 || t < best_t) { best_t = t; best = tile + NUM_TILES * si; }
-        }
-    }
+    const int best = select_staged(dtype, m, n, k, batch);
     // ring configs: same tile geometry, deeper prefetch, no edge handling.  Where one applies it replaces the
     // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).  For fp16 the ring
     // kernel on 16x16 MFMA blocks takes its place (faster than both the 32x32x16 ring and the wide-unit kernel on
@@ -459,9 +484,30 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     const double beta_d = f64 ? *static_cast<const double *>(beta) : (double)*static_cast<const float *>(beta);
     const float alpha_f = (float)alpha_d, beta_f = (float)beta_d;
 
+    const size_t esz_in = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
     if (config_id == MMBO_CONFIG_AUTO) {
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
+        // The pick is made from the shape alone.  The whole-tile kernels also need 16-byte aligned A and B and a
+        // tile's span of an operand below 2 GiB: where the operands at hand do not qualify, the staged kernel
+        // (any alignment) takes the call.
+        if (!f64) {
+            const ConfigRef c = config_ref(config_id);
+            if (c.ring) {
+                auto al16 = [&](const void *p, size_t ld, long long stride) {
+                    return ((uintptr_t)p % 16 == 0) && ((ld * esz_in) % 16 == 0) && (((size_t)stride * esz_in) % 16 == 0);
+                };
+                if (!al16(A, lda, strideA) || !al16(B, ldb, strideB)) config_id = select_staged(dtype, m, n, k, batch);
+            }
+        }
+        if (!tile_span_ok(config_tile(dtype, config_id), transA, transB, lda, ldb, esz_in)) {
+            // enormous leading dimensions: the first staged tile (no split-K) whose span fits, large tiles first
+            const int ntiles = f64 ? NUM_F64_TILES : NUM_TILES;
+            config_id = -1;
+            for (int tile = 0; tile < ntiles && config_id < 0; ++tile)
+                if (tile_span_ok(config_tile(dtype, tile), transA, transB, lda, ldb, esz_in)) config_id = tile;
+            if (config_id < 0) return MMBO_ERR_INVALID_SIZE;
+        }
     }
     const ConfigRef cref = f64 ? ConfigRef{false, config_id, 1} : config_ref(config_id);
     const size_t esz = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
@@ -472,12 +518,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
-    // per-thread global offsets are 32-bit: one tile's span of an operand must stay below 2 GiB
-    {
-        size_t span_a = (transA ? (size_t)r.bm : (size_t)r.bk) * lda * esz;
-        size_t span_b = (transB ? (size_t)r.bk : (size_t)r.bn) * ldb * esz;
-        if (span_a >= 0x7FFFFF00ull || span_b >= 0x7FFFFF00ull) return MMBO_ERR_INVALID_CONFIG;
-    }
+    if (!tile_span_ok(r, transA, transB, lda, ldb, esz)) return MMBO_ERR_INVALID_CONFIG;
 
     size_t nwg0 = ceil_div(m, r.bm), nwg1 = ceil_div(n, r.bn);
     if (nwg0 * nwg1 > 0x7FFFFFFFull) return MMBO_ERR_INVALID_SIZE;

@@ -446,3 +446,45 @@ def test_offline_tuner_emits_table_rows_for_small_shapes():
         m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), ([\d.]+)f\},", row)
         assert m and tuple(int(x) for x in m.groups()[:7]) == s[:7]
         assert 0 <= int(m.group(8)) < G.num_configs(s[0]) and float(m.group(9)) > 0
+
+
+def test_automatic_pick_never_fails_on_its_own_choice():
+    """MMBO_CONFIG_AUTO picks from the shape; the whole-tile kernels also need 16-byte aligned A and B and a tile span
+    below 2 GiB.  With operands that do not qualify the call must still succeed (staged kernel), while naming the
+    whole-tile config explicitly is refused."""
+    import torch
+
+    import gemm_mmbo_amd as G
+    # a whole-tile shape whose pick is a direct-to-LDS config, A (then B) one element off 16-byte alignment
+    for dtype in (F16, F32):
+        m, n, k = 1024, 1024, 512
+        cid = G.select_config(dtype, 0, 0, m, n, k)
+        assert "DTL1" in G.config_info(dtype, cid)["name"]
+        for offs in ((1, 0, 0), (0, 1, 0)):
+            p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=90, dist="normal" if dtype == F16 else "uniform", c_fill="nan")
+            with pytest.raises(G.MmboError) as e:
+                U.run_gpu(p, cid, offs)
+            assert e.value.status == 5
+            _run_and_check(p, -1, label=f"auto with unaligned operand {offs}", offsets=offs)
+    # a leading dimension so large that the rows of A^T under the picked tile span more than 2 GiB (only the first k rows of
+    # each stored column are used): the pick itself is refused by name, the automatic path moves to a tile that fits
+    m, n, k = 64, 16384, 100
+    pick = G.select_config(F32, 1, 0, m, n, k)
+    tm = G.config_info(F32, pick)["macro_tile_m"]
+    assert tm >= 64                                             # a smaller tile exists to fall back to
+    lda = 2 ** 31 // (tm * 4) + 4096                            # tm rows of A^T span just over 2 GiB (A: 2.1 GB at tm = 64)
+    rng = np.random.default_rng(91)
+    hA = rng.uniform(-1, 1, (m, k)).astype(np.float32)          # row i = the k values of column i of the stored k x m matrix
+    hB = rng.uniform(-1, 1, (n, k)).astype(np.float32)          # B stored k x n, column j = hB[j]
+    dA = torch.zeros(m * lda, dtype=torch.float32, device="cuda")
+    dA.view(m, lda)[:, :k] = torch.from_numpy(hA).cuda()
+    dB = torch.from_numpy(hB.reshape(-1)).cuda()
+    dC = torch.full((m * n,), float("nan"), dtype=torch.float32, device="cuda")
+    with pytest.raises(G.MmboError) as e:
+        G.gemm(F32, 1, 0, m, n, k, 1.0, dA, lda, dB, k, 0.0, dC, m, pick)
+    assert e.value.status == 5
+    G.gemm(F32, 1, 0, m, n, k, 1.0, dA, lda, dB, k, 0.0, dC, m, -1)
+    torch.cuda.synchronize()
+    want = hA.astype(np.float64) @ hB.astype(np.float64).T
+    got = dC.cpu().numpy().reshape((m, n), order="F")
+    assert np.max(np.abs(got - want)) <= U.tol(F32, k) * max(np.max(np.abs(want)), 1.0)
