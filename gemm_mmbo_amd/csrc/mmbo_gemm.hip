@@ -344,6 +344,44 @@ static bool tile_span_ok(const TileRow &r, int transA, int transB, size_t lda, s
     return span_a < 0x7FFFFF00ull && span_b < 0x7FFFFF00ull;
 }
 
+// Modelled time, in microseconds, of a whole-tile kernel (ring or x16 family, ring tile index rt: 256x256, 128x128,
+// 128x64, 64x64) on a shape made of whole tiles.  Work-groups run in rounds of (CUs x work-groups per CU); a tile costs
+// a ring fill, its slices at the family's in-loop efficiency (shared by the work-groups resident on the CU) and its
+// C traffic; the last, partial round runs with fewer work-groups per CU; split-K adds the reduction launch.  The
+// constants are a least-squares fit to the times of every such config on 45 shapes (gemm_mmbo_amd/tune.py --dump);
+// on those shapes the model's pick is within 2.5 % of the fastest config on average, 21 % at worst.
+static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, size_t n, size_t k, int batch)
+{
+    static const double eff[2][2][NUM_RING_TILES] = {
+        // 256x256 128x128 128x64  64x64
+        {{0.9451, 0.9134, 0.8667, 0.9015}, {0.9387, 0.9039, 0.8402, 0.8561}},       // fp32: ring, x16
+        {{0.5607, 0.3426, 0.2795, 0.2658}, {0.5879, 0.4873, 0.3151, 0.2560}},       // fp16: ring, x16
+    };
+    const double launch = 5.9, fill = 0.65, c_us_per_kb = 0.0272, reduce_launch = 1.43, reduce_us_per_mb = 0.28;
+    const RingRow &r = kRingTiles[rt];                     // the x16 tiles of the same macro tile have the same depth
+    const double esz = dtype == MMBO_F32 ? 4.0 : 2.0;
+    const double flop_per_us_cu = dtype == MMBO_F32 ? 0.614e6 : 9.83e6;             // matrix peak of one CU
+    const int bk = ring_bk(dtype);
+    const int lds = r.depth * (r.bm + r.bn) * 64;
+    int per_cu = 160 * 1024 / lds;
+    if (per_cu > 3) per_cu = 3;
+    if (per_cu < 1) per_cu = 1;
+    const double cus = 256.0;
+    const double wgs = (double)(m / r.bm) * (double)(n / r.bn) * split * batch;
+    const double slices = (double)(k / split) / bk;
+    const double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
+    auto tile_time = [&](double resident) {
+        return fill + slices * (2.0 * r.bm * r.bn * bk / flop_per_us_cu) * resident / e +
+               c_us_per_kb * r.bm * r.bn * esz * resident / 1e3;
+    };
+    const double slots = cus * per_cu;
+    const double full = std::floor(wgs / slots), last = wgs - full * slots;
+    double t = launch + full * tile_time(per_cu);
+    if (last > 0) t += tile_time(std::ceil(last / cus));
+    if (split > 1) t += reduce_launch + reduce_us_per_mb * (double)m * n * batch * (split * 4.0 + esz) / 1e6;
+    return t;
+}
+
 // The cost model's pick among the staged configs (fp32/fp16), which take any shape and any alignment.
 static int select_staged(int dtype, size_t m, size_t n, size_t k, int batch)
 {
@@ -384,31 +422,30 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
             t.batch == batch)
             return t.config_id;
-    const int best = select_staged(dtype, m, n, k, batch);
-    // ring configs: same tile geometry, deeper prefetch, no edge handling.  Where one applies it replaces the
-    // staged pick of the same or larger tile (measured faster on every whole-tile shape tried).  For fp16 the ring
-    // kernel on 16x16 MFMA blocks takes its place (faster than both the 32x32x16 ring and the wide-unit kernel on
-    // every shape swept).
+    // Whole-tile kernels (deeper prefetch, no edge handling) measured faster than the staged kernel on every shape
+    // they apply to: where one applies, the fastest of them by model_time_ring takes the call.  fp16: the x16 family
+    // (16x16x32 MFMAs), except that the 64 x 64 tile is faster on 32x32x16; fp32: the ring family, except that the
+    // x16 kernel's 256 x 256 tile (v_mfma_f32_16x16x4_f32, four wavefronts) measures 1.5-2 % faster than the ring
+    // kernel's at 8192^3 in NN, TN and TT (0.8 % slower in NT).
     {
-        const ConfigRef c = config_ref(best);
-        const TileRow &t = tile_row(dtype, c.tile);
         static const int x16_of_ring[NUM_RING_TILES] = {0, 2, 3, 4};       // same macro tile in kX16Tiles (256 x 256: four wavefronts)
-        for (int rt = 0; rt < NUM_RING_TILES; ++rt) {
-            const RingRow &r = kRingTiles[rt];
-            if (r.bm * r.bn > t.bm * t.bn) continue;
-            for (int si = 0; si < NUM_SPLITS; ++si)
-                if (kSplits[si] == c.split && ring_shape_ok(dtype, rt, c.split, m, n, k))
-                {
-                    if (dtype == MMBO_F16) return x16_config_id(x16_of_ring[rt], si);
-                    // fp32: the x16 kernel's 256 x 256 tile (v_mfma_f32_16x16x4_f32, four wavefronts) measures 1.5-2 %
-                    // faster than the ring kernel's at 8192^3 in NN, TN and TT and 0.8 % slower in NT; the smaller
-                    // tiles are equal within noise and stay with the ring kernel
-                    if (rt == 0 && !(transA == 0 && transB == 1)) return x16_config_id(0, si);
-                    return ring_config_id(rt, si);
+        int pick = -1;
+        double pick_t = 0.0;
+        for (int rt = 0; rt < NUM_RING_TILES; ++rt)
+            for (int si = 0; si < NUM_SPLITS; ++si) {
+                if (!ring_shape_ok(dtype, rt, kSplits[si], m, n, k)) continue;
+                if (kSplits[si] > 1 && (k / ring_bk(dtype)) / (size_t)kSplits[si] < 2) continue;      // slices too thin
+                if ((size_t)batch * kSplits[si] > 65535) continue;
+                const bool x16 = dtype == MMBO_F16 ? rt != 3 : (rt == 0 && !(transA == 0 && transB == 1));
+                const double t = model_time_ring(dtype, x16, rt, kSplits[si], m, n, k, batch);
+                if (pick < 0 || t < pick_t) {
+                    pick_t = t;
+                    pick = x16 ? x16_config_id(x16_of_ring[rt], si) : ring_config_id(rt, si);
                 }
-        }
+            }
+        if (pick >= 0) return pick;
     }
-    return best;
+    return select_staged(dtype, m, n, k, batch);
 }
 
 int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,

@@ -8,6 +8,7 @@ GPU it runs on:
     python -m gemm_mmbo_amd.tune                      # the built-in shape list (benchmark configs + HPL sweep points)
     python -m gemm_mmbo_amd.tune shapes.txt           # one shape per line:  dtype ta tb m n k batch alpha beta
                                                       # (dtype 0 fp32, 1 fp16, 2 fp64; ta/tb 0 = N, 1 = T)
+    python -m gemm_mmbo_amd.tune shapes.txt --dump t.json    # also write every config's time per shape
 
 For every shape it prints the ranking and one line in the table's syntax; paste the lines into kTuned[] and rebuild.
 Configs that do not apply to a shape (whole-tile kernels on ragged shapes) are skipped, as the C ABI refuses them.
@@ -57,13 +58,13 @@ def time_config(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, cfg, reps)
     return e0.elapsed_time(e1) / reps
 
 
-def tune(shapes, out=sys.stdout):
+def tune(shapes, out=sys.stdout, dump=None):
     import torch
 
     import gemm_mmbo_amd as G
     if not torch.cuda.is_available():
         raise RuntimeError("the tuner times kernels: it needs the GPU")
-    rows = []
+    rows, table = [], []
     for (dtype, ta, tb, m, n, k, batch, alpha, beta) in shapes:
         flops = 2.0 * m * n * k * batch
         reps = 3 if flops > 1e11 else 20
@@ -86,18 +87,29 @@ def tune(shapes, out=sys.stdout):
               f"({'%.1f us' % (t_pick * 1e3) if t_pick else 'not timed'}); fastest: "
               + "  ".join(f"{c} {G.config_info(dtype, c)['name']} {t * 1e3:.1f} us" for t, c in res[:4]), file=out)
         print(row, file=out, flush=True)
+        table.append({"shape": [dtype, ta, tb, m, n, k, batch, alpha, beta], "pick": pick,
+                      "ms": {str(c): t for t, c in res}})
+    if dump:
+        import json
+        with open(dump, "w") as f:
+            json.dump(table, f)
     return rows
 
 
 def main(argv):
     shapes = BUILTIN
+    dump = None
+    if "--dump" in argv:                      # every config's time per shape, as JSON
+        i = argv.index("--dump")
+        dump = argv[i + 1]
+        argv = argv[:i] + argv[i + 2:]
     if len(argv) > 1:
         shapes = []
         for line in open(argv[1]):
             f = line.split("#")[0].split()
             if f:
                 shapes.append(tuple(int(x) for x in f[:7]) + (float(f[7]), float(f[8])))
-    tune(shapes)
+    tune(shapes, dump=dump)
 
 
 if __name__ == "__main__":
