@@ -100,6 +100,16 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out);
  * negative mmbo_status on bad arguments.  Pure host logic: needs no device. */
 int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch);
 
+/* What MMBO_CONFIG_AUTO does with a large problem whose M or N is not a whole number of tiles (and whose A and B are
+ * 16-byte aligned): the block [0, m0) x [0, n0), cut at tile multiples, goes to a whole-tile kernel, the columns
+ * n0 .. n and the rows m0 .. m of the first n0 columns go to the staged kernel in up to two further launches on the
+ * same stream; every element of C is written by exactly one of them.  Returns 1 and the cut when the rule applies to
+ * the shape, 0 (and m0 = m, n0 = n) when the call is a single launch, a negative mmbo_status on bad arguments.  The
+ * reference's kernels take whole tiles only (src/gemm/ref/Kernels.cpp:153-1123 has no edge handling).  Pure host
+ * logic: needs no device. */
+int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
+                            size_t *n0);
+
 /* Host twin of the kernels' work-group -> tile mapping: linear work-group id to (tile row, tile
  * column).  With num_xcd = 1 and linear_id = wg0 + wg1*nwg0 this is the reference's
  * WorkGroupMapping remap (src/gemm/ref/Kernels.cpp:204-236, src/gemm/ref/map.cpp:11-38);

@@ -488,3 +488,25 @@ def test_automatic_pick_never_fails_on_its_own_choice():
     want = hA.astype(np.float64) @ hB.astype(np.float64).T
     got = dC.cpu().numpy().reshape((m, n), order="F")
     assert np.max(np.abs(got - want)) <= U.tol(F32, k) * max(np.max(np.abs(want)), 1.0)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_large_ragged_problems_are_cut_into_block_and_strips(dtype):
+    """MMBO_CONFIG_AUTO on shapes mmbo_auto_decomposition applies to: a whole-tile block and up to two strips, every
+    element of C written once; against the oracle, with beta, ld > dim (padding rows untouched), every transpose, a
+    batch, and bit-identical on repetition."""
+    import gemm_mmbo_amd as G
+    dist = "normal" if dtype == F16 else "uniform"
+    cases = [(0, 0, 2100, 2300, 2560, 1.0, 0.0, {}), (0, 1, 2100, 2048, 2560, -1.0, 1.0, {}), (1, 0, 2048, 2100, 2560, 1.5, 0.5, {}),
+             (1, 1, 1500, 1900, 4096, 1.0, 0.0, {}), (0, 0, 2100, 2300, 2560, 1.0, 1.0, {"lda": 2104, "ldb": 2568, "ldc": 2111}),
+             (0, 1, 1200, 1300, 2304, 1.0, 0.5, {"batch": 3})]
+    for (ta, tb, m, n, k, alpha, beta, kw) in cases:
+        batch = kw.get("batch", 1)
+        assert G.auto_decomposition(dtype, ta, tb, m, n, k, batch) is not None
+        p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, seed=500 + m + n, dist=dist, c_fill="uniform" if beta else "nan", **kw)
+        got = _run_and_check(p, -1, label=f"decomposed {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} {kw}")
+        again, _ = U.run_gpu(p, -1)
+        assert np.array_equal(got.view(U.BITS[dtype]), again.view(U.BITS[dtype]))
+    # unaligned A: the rule's shape applies, the operands do not: one staged launch, same result bar
+    p = U.Problem(dtype, 0, 0, 2100, 2300, 2560, 1.0, 0.0, seed=77, dist=dist, c_fill="nan")
+    _run_and_check(p, -1, label="ragged, unaligned A", offsets=(1, 0, 0))
