@@ -214,6 +214,29 @@ def main():
         del tensors, host
         torch.cuda.empty_cache()
 
+    # The same HGEMM on constant operands (all ones): the matrix pipes then draw far less power and the clock stays up,
+    # which separates what the kernel's structure costs from what the chip's power limit costs on real data.
+    ones_tflops = None
+    if not args.only:
+        A1 = torch.ones(m * k, device="cuda", dtype=torch.float16)
+        B1 = torch.ones(k * n, device="cuda", dtype=torch.float16)
+        C1 = torch.empty(m * n, device="cuda", dtype=torch.float16)
+        st = torch.cuda.current_stream()
+        cid1 = G.select_config(G.F16, 0, 0, m, n, k, 1)
+        for _ in range(5):
+            G.gemm(G.F16, G.OP_N, G.OP_N, m, n, k, 1.0, A1, m, B1, k, 0.0, C1, m, cid1, st)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(st)
+        for _ in range(20):
+            G.gemm(G.F16, G.OP_N, G.OP_N, m, n, k, 1.0, A1, m, B1, k, 0.0, C1, m, cid1, st)
+        e1.record(st)
+        torch.cuda.synchronize()
+        ones_tflops = flops / (e0.elapsed_time(e1) / 20) * 1e-9
+        assert float(C1[12345]) == float(k)          # 8192 ones: exact in fp16
+        del A1, B1, C1
+        torch.cuda.empty_cache()
+
     f64 = dgemm_legs(G, torch, args.steps, args.warmup) if args.only in (None, "f64") else {}
     skinny = skinny_legs(G, torch, args.steps, args.warmup) if not args.only else {}
     if args.only == "f64":
@@ -258,6 +281,9 @@ def main():
                        "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
                        "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
                        "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}
+    if ones_tflops is not None:
+        out.setdefault("also", {})["fp16_constant_operands_tflops"] = round(ones_tflops, 1)
+        out["also"]["fp16_constant_operands_frac_of_peak"] = round(ones_tflops / PEAK_TFLOPS["f16"], 4)
     if skinny:
         out.setdefault("also", {})["skinny_nn_hbm_bound"] = skinny
     if f64:
