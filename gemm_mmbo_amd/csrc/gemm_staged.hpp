@@ -64,7 +64,7 @@ struct OperandTile {
     // straddle the matrix edge or the end of K go element by element.
     typedef u32x4 __attribute__((aligned(2))) u32x4_unaligned;
     __device__ static inline void load_slow(u32x4 (&regs)[NCH], const char *g, const uint32_t (&off)[NCH],
-                                            int tid, uint32_t ld, int rows, int kvalid, bool vec)
+                                            int tid, uint32_t /* ld: the offsets already contain it */, int rows, int kvalid, bool vec)
     {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {

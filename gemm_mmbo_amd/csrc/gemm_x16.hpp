@@ -249,7 +249,8 @@ gemm_x16_kernel(const GemmArgs args)
     using TileB = typename Cfg::TileB;
     using FragA = typename Cfg::FragA;
     using FragB = typename Cfg::FragB;
-    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC, ESZ = Cfg::ESZ, MPF = Cfg::MPF;
+    constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC, ESZ = Cfg::ESZ;
+    [[maybe_unused]] constexpr int MPF = Cfg::MPF;
 
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 

@@ -603,7 +603,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
             if (config_id < 0) return MMBO_ERR_INVALID_SIZE;
         }
     }
-    const ConfigRef cref = f64 ? ConfigRef{false, config_id, 1} : config_ref(config_id);
+    const ConfigRef cref = f64 ? ConfigRef{false, config_id, 1, false} : config_ref(config_id);
     const size_t esz = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
     int split = cref.split;
     const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
