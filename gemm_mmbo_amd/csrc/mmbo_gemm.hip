@@ -3,6 +3,7 @@
 // layer src/gemm/gemm.h (front-ends), src/gemm/constants.h (tables) and src/gemm/driver.h (launch).
 #include "../../include/mmbo_gemm.h"
 
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -199,30 +200,25 @@ double model_time(int dtype, int tile, int split, size_t m, size_t n, size_t k, 
     return t;
 }
 
-// fp64: same model, one stage of prefetch, 64 MACs per clock per CU, no split-K.
+// fp64: microseconds.  Work-groups run in rounds of (CUs x work-groups per CU); a tile costs a fixed overhead
+// (first stage, C update, dispatch of its successor: measured per tile and CU with K swept from 96 to 1536 on the
+// HPL shape's M and N) plus its K at the tile's in-loop efficiency (from 8192^3), both shared by the work-groups
+// resident on the CU; the last, partial round runs with fewer of them.
 double model_time_f64(int tile, size_t m, size_t n, size_t k, int batch)
 {
+    //                                    128x128/4w 256x128/8w 64x64  32x32  128x128/8w 128x64
+    static const double overhead_us[NUM_F64_TILES] = {12.8, 26.5, 1.54, 0.25, 10.6, 5.9};
+    static const double in_loop_eff[NUM_F64_TILES] = {0.89, 0.853, 0.846, 0.704, 0.91, 0.84};
+    static const int resident[NUM_F64_TILES] = {2, 1, 5, 8, 2, 3};
     const TileRow &r = kTilesF64[tile];
-    const double cus = 256.0, mac_per_clk_cu = 64.0, hbm_bytes_per_clk = 3300.0, load_latency = 1700.0;
-    double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch;
-    int lds = dgemm_lds_bytes_of<0>(tile);
-    int per_cu = 160 * 1024 / (lds > 0 ? lds : 1);
-    int thr = r.wm * r.wn * 64;
-    if (per_cu > 1024 / thr) per_cu = 1024 / thr;      // the large tiles need more than 128 registers per lane
-    if (per_cu < 1) per_cu = 1;
-    double slots = cus * per_cu;
-    double rounds = (double)ceil_div((size_t)tiles, (size_t)slots);
-    double resident = tiles >= slots ? per_cu : (tiles > cus ? tiles / cus : 1.0);
-    double wave_cost = r.bm * r.bn / (r.wm * r.wn) >= 64 * 64 ? 1.0 : (r.bm >= 64 ? 1.1 : 1.5);
-    double stage_mfma = (double)r.bm * r.bn * r.bk * wave_cost / mac_per_clk_cu;
-    double stage = stage_mfma * resident > load_latency ? stage_mfma * resident : load_latency;
-    double stages = (double)ceil_div(k ? k : 1, (size_t)r.bk);
-    double epilogue = (double)r.bm * r.bn * 8.0 * resident / 24.0;
-    if (per_cu * thr >= 1024) epilogue *= 0.6;          // four wavefronts per SIMD hide part of the C traffic
-    double compute = rounds * (stages * stage + load_latency + epilogue);
-    double bytes = ((double)m * k + (double)k * n + (double)m * n) * batch * 8.0;
-    double t = compute > bytes / hbm_bytes_per_clk ? compute : bytes / hbm_bytes_per_clk;
-    return t + 9000.0;
+    const double cus = 256.0, flop_per_us_cu = 78.6e6 / 256.0, launch = 5.0;
+    const double tiles = (double)ceil_div(m, r.bm) * (double)ceil_div(n, r.bn) * batch;
+    const double per_tile = overhead_us[tile] + 2.0 * r.bm * r.bn * (double)(k ? k : 1) / flop_per_us_cu / in_loop_eff[tile];
+    const double slots = cus * resident[tile];
+    const double full = std::floor(tiles / slots), last = tiles - full * slots;
+    double t = launch + full * per_tile * resident[tile];
+    if (last > 0) t += per_tile * std::ceil(last / cus);
+    return t;
 }
 
 }  // namespace

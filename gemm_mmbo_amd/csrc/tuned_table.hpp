@@ -35,7 +35,7 @@ constexpr TunedRow kTuned[] = {
     {1, 0, 0, 8192, 8192, 8192, 1, 51, 1330.0f},
     {0, 0, 0, 4096, 4096, 4096, 1, 51, 143.6f},
     {1, 0, 0, 4096, 4096, 4096, 1, 51, 1245.0f},
-    {2, 0, 1, 44160, 2048, 384, 1, 4, 58.2f},      // the reference's HPL trailing update (src/gemm/run.sh:2-5)
+    {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // the reference's HPL trailing update (src/gemm/run.sh:2-5)
     {2, 0, 0, 8192, 8192, 8192, 1, 0, 69.7f},
 };
 

@@ -71,9 +71,10 @@ def test_select_config_headline_and_skinny_shapes():
     d = G.config_info(G.F32, G.select_config(G.F32, 0, 0, 40, 40, 64))
     assert d["macro_tile_m"] <= 64 and d["split_k"] == 1
     assert G.select_config(G.F32, 0, 0, 0, 5, 5) == 0
-    # fp64 has its own table: the reference's HPL trailing update gets a large tile, a tiny problem a small one
+    # fp64 has its own table: the reference's HPL trailing update gets the tile its sweep found fastest (with K = 384
+    # the 64 x 64 tile, five work-groups to a CU, edges out the 128 x 128 ones), a tiny problem a small one
     hpl = G.config_info(G.F64, G.select_config(G.F64, 0, 1, 44160, 2048, 384))
-    assert hpl["macro_tile_m"] * hpl["macro_tile_n"] >= 128 * 128 and hpl["split_k"] == 1
+    assert hpl["macro_tile_m"] * hpl["macro_tile_n"] >= 64 * 64 and hpl["split_k"] == 1
     assert G.config_info(G.F64, G.select_config(G.F64, 0, 1, 40, 40, 64))["macro_tile_m"] <= 64
     with pytest.raises(G.MmboError):
         G.select_config(3, 0, 0, 1, 1, 1)
