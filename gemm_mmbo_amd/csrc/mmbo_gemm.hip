@@ -444,9 +444,10 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
     return select_staged(dtype, m, n, k, batch);
 }
 
-// Large problems whose M or N is not a whole number of tiles: the whole-tile kernels are 2-3 times faster than
-// the staged kernel on the part they can take (measured: HGEMM 3072^3 68 us, 3000^3 through the staged kernel
-// 150 us).  Rule: fp32/fp16, k a whole number of ring slices, both m and n at least 512, at least 20 GFLOP (below
+// Large problems that are not made of whole tiles: the whole-tile kernels are 2-3 times faster than the staged
+// kernel on the part they can take (measured: HGEMM 3072^3 68 us, 3000^3 through the staged kernel 150 us).
+//
+// M and N.  Rule: fp32/fp16, k a whole number of ring slices, both m and n at least 512, at least 20 GFLOP (below
 // that the two extra launches cost more than the block gains: 2000 x 2000 x 512 measured twice as slow cut up), and
 // m or n not a multiple of 64 (otherwise a whole-tile kernel takes the whole problem anyway).  The block is cut at
 // multiples of 128 (64 below 1024).  Measured cut up against one staged launch: HGEMM 8200 x 8200 x 8192 1.70 x,
@@ -464,15 +465,37 @@ static bool auto_decomposition(int dtype, size_t m, size_t n, size_t k, int batc
     return true;
 }
 
+// K.  A k that is not a whole number of ring slices keeps a large problem off the whole-tile kernels altogether.
+// Rule: same element types, m and n at least 2048, k at least 1024, at least 20 GFLOP: the last k % slice columns of A
+// and rows of B go through the staged kernel first (C1 = alpha*A_tail*B_tail + beta*C, one pass over C), the first
+// k0 through MMBO_CONFIG_AUTO again as C = alpha*A0*B0 + 1*C1.  C1 is stored in C's element type: an fp16 result
+// is then rounded twice (fp32: the extra rounding is below the accumulation error).  Measured against one staged
+// launch: HGEMM 7000^3 TN 1.65 x, 8192 x 8192 x 8200 1.16 x, 2048 x 2048 x 3000 1.11 x, 3000^3 1.04 x; SGEMM 4100^3 NT
+// 2.0 x, 3000^3 1.19 x (1024 x 1024 x 10000 would lose 10 %: below the size limit).  Tightly packed operands with a
+// ragged leading dimension (NN with ldb = k) are not 16-byte aligned per column and stay with the staged kernel.
+static bool auto_k_split(int dtype, size_t m, size_t n, size_t k, int batch, size_t *k0)
+{
+    if (dtype != MMBO_F32 && dtype != MMBO_F16) return false;
+    const size_t bk = (size_t)ring_bk(dtype);
+    if (k < 1024 || k % bk == 0) return false;
+    if (m < 2048 || n < 2048) return false;
+    if (2.0 * (double)m * (double)n * (double)k * (double)(batch > 0 ? batch : 1) < 2e10) return false;
+    *k0 = k / bk * bk;
+    return true;
+}
+
 int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                            size_t *n0)
+                            size_t *n0, size_t *k0)
 {
     if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
     if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
-    if (!m0 || !n0) return -MMBO_ERR_NULL_POINTER;
+    if (!m0 || !n0 || !k0) return -MMBO_ERR_NULL_POINTER;
     *m0 = m;
     *n0 = n;
-    return auto_decomposition(dtype, m, n, k, batch, m0, n0) ? 1 : 0;
+    *k0 = k;
+    const bool ks = auto_k_split(dtype, m, n, k, batch, k0);
+    const bool mn = auto_decomposition(dtype, m, n, *k0, batch, m0, n0);
+    return ks || mn ? 1 : 0;
 }
 
 int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
@@ -552,10 +575,23 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (config_id == MMBO_CONFIG_AUTO) {
         // A large problem with ragged M or N: a whole-tile block plus up to two edge strips, each C element written
         // by exactly one of the launches (A and B must qualify for the whole-tile kernels, or nothing is gained).
-        size_t m0 = 0, n0 = 0;
-        if (auto_decomposition(dtype, m, n, k, batch, &m0, &n0) && (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 &&
-            (lda * esz_in) % 16 == 0 && (ldb * esz_in) % 16 == 0 && ((size_t)strideA * esz_in) % 16 == 0 &&
-            ((size_t)strideB * esz_in) % 16 == 0) {
+        size_t m0 = 0, n0 = 0, k0 = 0;
+        const bool whole_tile_operands = (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 && (lda * esz_in) % 16 == 0 &&
+                                         (ldb * esz_in) % 16 == 0 && ((size_t)strideA * esz_in) % 16 == 0 &&
+                                         ((size_t)strideB * esz_in) % 16 == 0;
+        if (whole_tile_operands && auto_k_split(dtype, m, n, k, batch, &k0)) {
+            // the K tail first, with the caller's beta; then the whole slices on top of it
+            const char *a8 = static_cast<const char *>(A), *b8 = static_cast<const char *>(B);
+            const size_t off_a = (transA ? k0 : k0 * lda) * esz_in, off_b = (transB ? k0 * ldb : k0) * esz_in;
+            int rc = mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k - k0, alpha, a8 + off_a, lda, strideA,
+                                               b8 + off_b, ldb, strideB, beta, C, ldc, strideC, batch,
+                                               select_staged(dtype, m, n, k - k0, batch), stream);
+            if (rc != MMBO_OK) return rc;
+            const float one = 1.0f;
+            return mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k0, alpha, A, lda, strideA, B, ldb, strideB, &one,
+                                             C, ldc, strideC, batch, MMBO_CONFIG_AUTO, stream);
+        }
+        if (whole_tile_operands && auto_decomposition(dtype, m, n, k, batch, &m0, &n0)) {
             const char *a8 = static_cast<const char *>(A), *b8 = static_cast<const char *>(B);
             char *c8 = static_cast<char *>(C);
             int rc = mmbo_gemm_strided_batched(dtype, transA, transB, m0, n0, k, alpha, A, lda, strideA, B, ldb, strideB,

@@ -211,18 +211,21 @@ def test_tuner_shape_list_is_valid_and_rows_parse():
 
 
 def test_auto_decomposition_rule():
-    """Large ragged problems are cut into a whole-tile block and edge strips; everything else is one launch."""
-    assert G.auto_decomposition(G.F16, 0, 0, 3000, 3000, 3008) == (2944, 2944)      # 23 x 128
-    assert G.auto_decomposition(G.F32, 1, 0, 1000, 4100, 4096) == (960, 4096)       # below 1024: cut at 64
-    assert G.auto_decomposition(G.F16, 0, 1, 4096, 4100, 4096) == (4096, 4096)      # only N ragged
-    assert G.auto_decomposition(G.F16, 0, 0, 3000, 3000, 3000) is None              # k not a whole number of slices
-    assert G.auto_decomposition(G.F32, 0, 0, 3000, 3000, 3000) is None
+    """Large problems that are not made of whole tiles are cut into a whole-tile block, edge strips and a K tail;
+    everything else is one launch."""
+    assert G.auto_decomposition(G.F16, 0, 0, 3000, 3000, 3008) == (2944, 2944, 3008)      # 23 x 128
+    assert G.auto_decomposition(G.F32, 1, 0, 1000, 4100, 4096) == (960, 4096, 4096)       # below 1024: cut at 64
+    assert G.auto_decomposition(G.F16, 0, 1, 4096, 4100, 4096) == (4096, 4096, 4096)      # only N ragged
+    assert G.auto_decomposition(G.F16, 0, 0, 3000, 3000, 3000) == (2944, 2944, 2976)      # and a K tail of 24
+    assert G.auto_decomposition(G.F32, 0, 0, 3000, 3000, 3000) == (2944, 2944, 2992)      # fp32 slices are 16 wide
+    assert G.auto_decomposition(G.F16, 1, 0, 4096, 4096, 4100) == (4096, 4096, 4096)      # only K ragged
     assert G.auto_decomposition(G.F16, 0, 0, 4096, 4096, 4096) is None              # already whole tiles
     assert G.auto_decomposition(G.F16, 0, 0, 1023, 777, 512) is None                # too little work
     assert G.auto_decomposition(G.F16, 0, 0, 2000, 2000, 512) is None
+    assert G.auto_decomposition(G.F16, 0, 0, 4096, 4096, 1000) is None              # K tail of a short K: not worth a pass over C
     assert G.auto_decomposition(G.F16, 0, 0, 400, 50000, 4096) is None              # a skinny side
     assert G.auto_decomposition(G.F64, 0, 1, 3000, 3000, 3008) is None              # fp64 has no whole-tile kernel
-    for (m, n, k) in ((3000, 3000, 3008), (1000, 4100, 4096)):
-        m0, n0 = G.auto_decomposition(G.F16, 0, 0, m, n, k)
-        assert m0 % 64 == 0 and n0 % 64 == 0 and m - m0 < 128 and n - n0 < 128
-        assert "DTL1" in G.config_info(G.F16, G.select_config(G.F16, 0, 0, m0, n0, k))["name"]
+    for (m, n, k) in ((3000, 3000, 3008), (1000, 4100, 4096), (3000, 3000, 3000)):
+        m0, n0, k0 = G.auto_decomposition(G.F16, 0, 0, m, n, k)
+        assert m0 % 64 == 0 and n0 % 64 == 0 and k0 % 32 == 0 and m - m0 < 128 and n - n0 < 128 and k - k0 < 32
+        assert "DTL1" in G.config_info(G.F16, G.select_config(G.F16, 0, 0, m0, n0, k0))["name"]

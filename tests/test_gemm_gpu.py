@@ -499,7 +499,10 @@ def test_large_ragged_problems_are_cut_into_block_and_strips(dtype):
     dist = "normal" if dtype == F16 else "uniform"
     cases = [(0, 0, 2100, 2300, 2560, 1.0, 0.0, {}), (0, 1, 2100, 2048, 2560, -1.0, 1.0, {}), (1, 0, 2048, 2100, 2560, 1.5, 0.5, {}),
              (1, 1, 1500, 1900, 4096, 1.0, 0.0, {}), (0, 0, 2100, 2300, 2560, 1.0, 1.0, {"lda": 2104, "ldb": 2568, "ldc": 2111}),
-             (0, 1, 1200, 1300, 2304, 1.0, 0.5, {"batch": 3})]
+             (0, 1, 1200, 1300, 2304, 1.0, 0.5, {"batch": 3}),
+             # K that is not a whole number of slices: a tail pass first, then the whole slices on top
+             (0, 0, 2104, 2304, 2568, 1.0, 0.0, {}), (1, 0, 2048, 2048, 3000, -1.0, 1.0, {}), (0, 1, 2048, 2304, 2570, 1.5, 0.5, {}),
+             (1, 1, 2056, 2048, 1208, 1.0, 0.5, {"batch": 2})]
     for (ta, tb, m, n, k, alpha, beta, kw) in cases:
         batch = kw.get("batch", 1)
         assert G.auto_decomposition(dtype, ta, tb, m, n, k, batch) is not None
