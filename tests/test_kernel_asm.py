@@ -41,7 +41,7 @@ def _compile(unit, outdir):
 
 
 def _kernels(path):
-    """{kernel symbol: list of instruction lines} of one assembly file."""
+    """{kernel symbol: list of instruction lines (and '.LBB..:' labels)} of one assembly file."""
     lines = open(path).read().split("\n")
     starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
     out = {}
@@ -52,7 +52,9 @@ def _kernels(path):
             t = l.strip()
             if t.startswith(".amdhsa_kernel") or t.startswith(".section"):
                 break
-            if t and not t.startswith(";") and not t.startswith("."):
+            if re.match(r"^\.LBB\w+:", t):
+                body.append(t.split(":")[0] + ":")
+            elif t and not t.startswith(";") and not t.startswith("."):
                 body.append(t.split(";")[0].strip())
         out[lines[i].split(":")[0]] = body
     return out
@@ -67,21 +69,43 @@ def _vregs(text):
 
 
 def _inflight_violations(body):
-    pending, bad = set(), []
-    for t in body:
-        m = re.match(r"ds_read\w* (v\[\d+:\d+\]|v\d+),", t)
+    """Forward data flow over the kernel's control-flow graph: the set of registers with an LDS read in flight at
+    each instruction is the union over its predecessors; a read adds its destination, `s_waitcnt lgkmcnt(0)` empties
+    the set, and any other instruction that names a register of the set is a violation."""
+    label = {t[:-1]: i for i, t in enumerate(body) if t.endswith(":")}
+
+    def succ(i, t):
+        if t.startswith("s_endpgm"):
+            return []
+        m = re.match(r"s_(c?branch\w*) (\.LBB\w+)", t)
         if m:
-            addr = _vregs(t[m.end():])
-            if addr & pending:
-                bad.append(t)
-            pending |= _vregs(m.group(1))
-            continue
-        if t.startswith("s_waitcnt") and "lgkmcnt(0)" in t:
-            pending = set()
-            continue
-        if pending and (_vregs(t) & pending):
-            bad.append(t)
-    return bad
+            tgt = label[m.group(2)]
+            return [tgt] if m.group(1) == "branch" else [i + 1, tgt]
+        return [i + 1] if i + 1 < len(body) else []
+
+    pend_in = [None] * len(body)
+    pend_in[0] = frozenset()
+    work, bad = [0], {}
+    while work:
+        i = work.pop()
+        t, cur = body[i], pend_in[i]
+        out = cur
+        if not t.endswith(":"):
+            m = re.match(r"ds_read\w* (v\[\d+:\d+\]|v\d+),", t)
+            if m:
+                if _vregs(t[m.end():]) & cur:
+                    bad[i] = t
+                out = cur | _vregs(m.group(1))
+            elif t.startswith("s_waitcnt") and "lgkmcnt(0)" in t:
+                out = frozenset()
+            elif cur and (_vregs(t) & cur):
+                bad[i] = t
+        for j in succ(i, t):
+            new = out if pend_in[j] is None else pend_in[j] | out
+            if new != pend_in[j]:
+                pend_in[j] = frozenset(new)
+                work.append(j)
+    return [bad[i] for i in sorted(bad)]
 
 
 @pytest.fixture(scope="module")
@@ -97,6 +121,13 @@ def test_checker_sees_a_planted_violation():
     ok = ["ds_read_b64_tr_b16 v[10:11], v5", "v_mfma_f32_16x16x32_f16 a[0:3], v[20:23], v[24:27], a[0:3]",
           "s_waitcnt vmcnt(2)", "s_waitcnt lgkmcnt(0)", "v_mfma_f32_16x16x32_f16 a[0:3], v[10:13], v[24:27], a[0:3]"]
     assert _inflight_violations(ok) == []
+    # control flow: the block after an unconditional branch is not its successor, the branch target is
+    jump = ["ds_read_b32 v7, v3", "s_branch .LBB0_2", ".LBB0_1:", "v_mov_b32_e32 v7, 0", "s_endpgm", ".LBB0_2:",
+            "s_waitcnt lgkmcnt(0)", "v_add_u32_e32 v8, v7, v7", "s_endpgm"]
+    assert _inflight_violations(jump) == []
+    loop = [".LBB0_1:", "v_add_u32_e32 v9, v7, v7", "ds_read_b32 v7, v3", "s_cbranch_scc1 .LBB0_1", "s_waitcnt lgkmcnt(0)",
+            "s_endpgm"]
+    assert _inflight_violations(loop) == ["v_add_u32_e32 v9, v7, v7"]       # the back edge carries the read in flight
 
 
 def test_no_register_is_touched_while_its_lds_read_is_in_flight(asm_files):
