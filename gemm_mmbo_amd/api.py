@@ -147,18 +147,17 @@ def select_config(dtype, transA, transB, m, n, k, batch=1):
 
 
 def auto_decomposition(dtype, transA, transB, m, n, k, batch=1):
-    """(m0, n0, k0) of the whole-tile block MMBO_CONFIG_AUTO cuts out of a large problem that is not made of whole
-    tiles, or None when the call is a single launch."""
+    """(m0, n0) of the block MMBO_CONFIG_AUTO cuts out of a large problem whose ragged M or N the fast kernels' edge
+    tiles cannot take, or None when the call is a single launch."""
     L = lib()
     L.mmbo_auto_decomposition.argtypes = [ctypes.c_int] * 3 + [ctypes.c_size_t] * 3 + [ctypes.c_int] + \
-        [ctypes.POINTER(ctypes.c_size_t)] * 3
+        [ctypes.POINTER(ctypes.c_size_t)] * 2
     L.mmbo_auto_decomposition.restype = ctypes.c_int
-    m0, n0, k0 = ctypes.c_size_t(0), ctypes.c_size_t(0), ctypes.c_size_t(0)
-    r = L.mmbo_auto_decomposition(dtype, transA, transB, m, n, k, batch, ctypes.byref(m0), ctypes.byref(n0),
-                                  ctypes.byref(k0))
+    m0, n0 = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    r = L.mmbo_auto_decomposition(dtype, transA, transB, m, n, k, batch, ctypes.byref(m0), ctypes.byref(n0))
     if r < 0:
         _check(-r)
-    return (m0.value, n0.value, k0.value) if r == 1 else None
+    return (m0.value, n0.value) if r == 1 else None
 
 
 def wg_remap(linear_id, nwg0, nwg1, wgm=8, num_xcd=8):

@@ -1,10 +1,10 @@
 // Ring kernel on 16 x 16 MFMA blocks (v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32) with the accumulators pinned
 // to the accumulation registers.
 //
-// Same structure as gemm_ring.hpp (whole tiles only; K in slices of 64 bytes per row -- 32 halves or 16 floats --
-// through a ring of LDS buffers filled by
-// global->LDS direct loads; fragments double-buffered in registers; one barrier per slice), and the same recipe
-// as the reference's kernels (src/gemm/ref/Kernels.cpp:412-747).  Two differences, both about energy: MI355X
+// Same structure as gemm_ring.hpp (K in slices of 64 bytes per row -- 32 halves or 16 floats -- through a ring of LDS
+// buffers filled by global->LDS direct loads; fragments double-buffered in registers; one barrier per slice), and the
+// same recipe as the reference's kernels (src/gemm/ref/Kernels.cpp:412-747).  Unlike gemm_ring.hpp it also takes
+// ragged problems: edge tiles load clamped rows and store under guards, a partial last slice of k is zero-filled.  Two differences, both about energy: MI355X
 // lowers its clock under the power that fp16 MFMAs on real data draw, so what a kernel costs per flop outside
 // the matrix pipe, and what the matrix instruction itself costs, decide the rate.
 //   - 16x16x32 blocks: measured on the same random operands a register-only loop of v_mfma_f32_16x16x32_f16
@@ -131,18 +131,58 @@ struct Tile {
     __device__ static inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ kc_swz(row)) << 4); }
     __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4); }
 
-    // global byte offset (from the tile origin of this slice) of the chunk that lands in LDS slot (wave*LPW + i)*64 + lane
-    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld)
+    // global byte offset (from the tile origin of this slice) of the chunk that lands in LDS slot (wave*LPW + i)*64 + lane.
+    // `valid` = rows of the tile that exist in the operand (R, or fewer for the last tile of a ragged dimension): the
+    // slots of the rows past the edge are filled with a copy of the last row (KC) or the last 16-byte group of rows
+    // (RC: the host guarantees that the dimension is a whole number of such groups) -- they only feed accumulators
+    // that are never stored, and every address stays inside the operand.
+    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld, uint32_t valid)
     {
         const uint32_t q = wave * LPW + i;
         if constexpr (KC) {
             uint32_t row = q * 16 + (lane >> 2);
             uint32_t chunk = (lane & 3) ^ kc_swz(row);
-            return row * ld * ESZ + chunk * 16;
+            return min(row, valid - 1) * ld * ESZ + chunk * 16;
         } else {
             uint32_t k = q * KPI + lane / CPR;
             uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-            return k * ld * ESZ + chunk * 16;
+            return k * ld * ESZ + min(chunk, valid * ESZ / 16 - 1) * 16;
+        }
+    }
+
+    // The last, partial slice of a k that is not a whole number of slices (reference: the tail loop,
+    // src/gemm/ref/Kernels.cpp:921-1005, zero-fills k >= remainder): the same slots as the direct loads fill, written
+    // through registers, with zeros from k_tail on.  g = operand origin of this tile at the tail slice.  Only elements
+    // that exist are read: a 16-byte chunk along k that straddles the end goes element by element.
+    __device__ static inline void fill_tail(const char *g, uint32_t ld, uint32_t valid, uint32_t k_tail, char *dst, int wave,
+                                            int lane)
+    {
+        constexpr uint32_t EPC = 16 / ESZ;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) {
+            const uint32_t q = wave * LPW + i;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if constexpr (KC) {
+                uint32_t row = q * 16 + (lane >> 2);
+                uint32_t chunk = (lane & 3) ^ kc_swz(row);
+                const char *p = g + min(row, valid - 1) * ld * ESZ + chunk * 16;
+                const uint32_t k0 = chunk * EPC;
+                if (k0 + EPC <= k_tail) {
+                    v = *reinterpret_cast<const u32x4 *>(p);
+                } else if (k0 < k_tail) {
+                    union { T e[EPC]; u32x4 v; } u;
+                    u.v = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                    for (uint32_t e = 0; e < EPC; ++e)
+                        if (k0 + e < k_tail) u.e[e] = reinterpret_cast<const T *>(p)[e];
+                    v = u.v;
+                }
+            } else {
+                uint32_t k = q * KPI + lane / CPR;
+                uint32_t chunk = (lane % CPR) ^ rc_mask(k);
+                if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + min(chunk, valid * ESZ / 16 - 1) * 16);
+            }
+            *reinterpret_cast<u32x4 *>(dst + q * 1024 + lane * 16) = v;
         }
     }
 };
@@ -276,8 +316,10 @@ gemm_x16_kernel(const GemmArgs args)
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
     const uint32_t lda = args.lda, ldb = args.ldb;
     const uint32_t k_begin = split * args.k_per_split;
-    const uint32_t k_end = min(args.k, k_begin + args.k_per_split);
+    // every split takes k_per_split (whole slices); the last one also the rest of k, whose last slice may be partial
+    const uint32_t k_end = split + 1 == args.splits ? args.k : min(args.k, k_begin + args.k_per_split);
     const int n_slice = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
+    const uint32_t k_tail = k_end > k_begin ? (k_end - k_begin) % BK : 0;
 
     const char *gA = static_cast<const char *>(args.A) +
                      ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda + k_begin
@@ -288,11 +330,13 @@ gemm_x16_kernel(const GemmArgs args)
     const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * ESZ;
     const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * ESZ;
 
+    // rows and columns of this tile that exist: less than the tile on the last tile row / column of a ragged problem
+    const uint32_t m_here = min((uint32_t)BM, args.m - row0), n_here = min((uint32_t)BN, args.n - col0);
     uint32_t offA[TileA::LPW], offB[TileB::LPW];
 #pragma unroll
-    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda);
+    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda, m_here);
 #pragma unroll
-    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb);
+    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here);
 
     // direct load number l (A's first, then B's) of slice s into ring buffer `buf`
     auto issue_load = [&](auto L, const char *pa, const char *pb, char *dst) {
@@ -566,6 +610,26 @@ gemm_x16_kernel(const GemmArgs args)
 #undef MMBO_WAIT_VM
 #undef MMBO_WAIT_LGKM0
 
+    if (k_tail != 0) {
+        // The partial last slice.  The loop ended on a barrier after every wavefront's last LDS read and with no load in
+        // flight, so buffer 0 is free: fill it through registers (zeros from k_tail on), then one more slice of MFMAs.
+        TileA::fill_tail(gA + (int64_t)n_slice * stepA, lda, m_here, k_tail, lds, wave, lane);
+        TileB::fill_tail(gB + (int64_t)n_slice * stepB, ldb, n_here, k_tail, lds + TileA::BYTES, wave, lane);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        fa[0].read_all(lds_base, adA);
+        fb[0].read_all(lds_base + TileA::BYTES, adB);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<Cfg::NMFMA>([&](auto M) {
+            constexpr int m = decltype(M)::value;
+            constexpr int tt = m / (FM * FN), ij = m % (FM * FN);
+            constexpr int i = ij / FN, j = (i & 1) ? FN - 1 - ij % FN : ij % FN;
+            if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(fa[0].x[i], fb[0].x[j]);
+            else mfma_acc_f32<(i * FN + j) * 4, NACC>(fa[0].x[i][tt], fb[0].x[j][tt]);
+        });
+        __syncthreads();            // the next tile's direct loads overwrite buffer 0
+    }
     if constexpr ((ABLATE & 8) != 0) t_probe[2] = wall_clock64();
     // the last MFMAs' results must have landed before they are read back
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
@@ -578,6 +642,53 @@ gemm_x16_kernel(const GemmArgs args)
     // when beta != 0 (reference: src/gemm/ref/Kernels.cpp:87); with GlobalSplitU > 1 the raw sums go to the fp32
     // workspace [split][batch][n][m] and the reduction kernel applies alpha and beta.
     const uint32_t wrow0 = row0 + wm * Cfg::TM + 4 * (lane >> 4), wcol0 = col0 + wn * Cfg::TN + (lane & 15);
+    if (m_here < (uint32_t)BM || n_here < (uint32_t)BN) {
+        // Edge tile (reference: the guarded store, src/gemm/ref/Kernels.cpp:1064-1121): every element is tested against
+        // m and n; four rows go out as one vector where all four exist and C allows it.
+        const float alpha = args.alpha, beta = args.beta;
+        const bool to_ws = args.splits > 1;
+        float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)args.m * args.n;
+        T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
+        const bool vec_c = args.vec_c != 0;
+        typedef typename std::conditional<ESZ == 2, u32x2, u32x4>::type cvec;
+        static_for<FM * FN>([&](auto IJ) {
+            constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
+            const uint32_t row = wrow0 + i * 16, col = wcol0 + j * 16;
+            float v[4] = {acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
+            if (col < args.n && row < args.m) {
+                if (to_ws) {
+                    float *p = ws + (size_t)col * args.m + row;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (row + r < args.m) p[r] = v[r];
+                } else {
+                    T *p = C + (size_t)col * args.ldc + row;
+                    if (vec_c && row + 3 < args.m) {
+                        union { T e[4]; cvec v; } io;
+                        if (beta != 0.0f) {
+                            io.v = *reinterpret_cast<const cvec *>(p);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], alpha * v[r]);
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) io.e[r] = (T)(alpha * v[r]);
+                        }
+                        *reinterpret_cast<cvec *>(p) = io.v;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            if (row + r < args.m) {
+                                float o = alpha * v[r];
+                                if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
+                                p[r] = (T)o;
+                            }
+                        }
+                    }
+                }
+            }
+        });
+        continue;
+    }
     if (args.splits > 1) {
         float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)args.m * args.n;
         static_for<FM * FN>([&](auto IJ) {

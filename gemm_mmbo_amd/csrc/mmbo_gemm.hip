@@ -51,12 +51,27 @@ inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_
     return dtype == MMBO_F16 && transA == transB && m % 256 == 0 && n % 256 == 0 && k % 64 == 0 && k >= 512;
 }
 
-inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k, bool x16 = false)
+// The x16 kernel takes ragged problems (its loads repeat the last rows of an edge tile, its edge tiles store under
+// guards, a partial last slice of k is zero-filled): only a dimension of op(A) or op(B) that is contiguous in memory
+// must be a whole number of 16-byte groups -- m under transA = N, n under transB = T.
+inline bool x16_edge_ok(int dtype, int transA, int transB, size_t m, size_t n)
+{
+    const size_t per16 = dtype == MMBO_F32 ? 4 : 8;
+    return (transA || m % per16 == 0) && (!transB || n % per16 == 0);
+}
+
+// Does the ring (x16 = false) or x16 config (tile, split) take this shape?  Ring: m, n whole tiles, k whole slices, the
+// same number for every split.  x16: whole tiles or x16_edge_ok; every split gets the same number of whole slices
+// (at least one when there is more than one split) and the last split the partial slice, if any.
+inline bool ring_shape_ok(int dtype, int tile, int split, int transA, int transB, size_t m, size_t n, size_t k, bool x16)
 {
     const RingRow &r = x16 ? kX16Tiles[tile] : kRingTiles[tile];
     const size_t bk = (size_t)ring_bk(dtype);
-    if (m % r.bm || n % r.bn || k == 0 || k % bk) return false;
-    return (k / bk) % (size_t)split == 0;          // every split gets the same whole number of slices
+    if (k == 0) return false;
+    const bool ragged = m % r.bm || n % r.bn || k % bk;
+    if (ragged && !(x16 && x16_edge_ok(dtype, transA, transB, m, n))) return false;
+    if (split > 1 && k / bk < (size_t)split) return false;
+    return (k / bk) % (size_t)split == 0;
 }
 
 thread_local int g_last_hip_error = 0;
@@ -363,8 +378,8 @@ static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, 
     if (per_cu > 3) per_cu = 3;
     if (per_cu < 1) per_cu = 1;
     const double cus = 256.0;
-    const double wgs = (double)(m / r.bm) * (double)(n / r.bn) * split * batch;
-    const double slices = (double)(k / split) / bk;
+    const double wgs = (double)ceil_div(m, (size_t)r.bm) * (double)ceil_div(n, (size_t)r.bn) * split * batch;
+    const double slices = std::ceil((double)k / bk) / split;
     const double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
     auto tile_time = [&](double resident) {
         return fill + slices * (2.0 * r.bm * r.bn * bk / flop_per_us_cu) * resident / e +
@@ -429,10 +444,16 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         double pick_t = 0.0;
         for (int rt = 0; rt < NUM_RING_TILES; ++rt)
             for (int si = 0; si < NUM_SPLITS; ++si) {
-                if (!ring_shape_ok(dtype, rt, kSplits[si], m, n, k)) continue;
+                const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], transA, transB, m, n, k, false);
+                const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], transA, transB, m, n, k, true);
+                if (!ring_ok && !x16_ok) continue;
+                // a dimension smaller than the tile stays with the staged kernel's smaller tiles
+                if (!ring_ok && (m < (size_t)kRingTiles[rt].bm || n < (size_t)kRingTiles[rt].bn)) continue;
                 if (kSplits[si] > 1 && (k / ring_bk(dtype)) / (size_t)kSplits[si] < 2) continue;      // slices too thin
                 if ((size_t)batch * kSplits[si] > 65535) continue;
-                const bool x16 = dtype == MMBO_F16 ? rt != 3 : (rt == 0 && !(transA == 0 && transB == 1));
+                bool x16 = dtype == MMBO_F16 ? rt != 3 : (rt == 0 && !(transA == 0 && transB == 1));
+                if (!ring_ok) x16 = true;           // ragged M or N: only the x16 kernel has edge tiles
+                if (!x16_ok) x16 = false;
                 const double t = model_time_ring(dtype, x16, rt, kSplits[si], m, n, k, batch);
                 if (pick < 0 || t < pick_t) {
                     pick_t = t;
@@ -444,58 +465,35 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
     return select_staged(dtype, m, n, k, batch);
 }
 
-// Large problems that are not made of whole tiles: the whole-tile kernels are 2-3 times faster than the staged
-// kernel on the part they can take (measured: HGEMM 3072^3 68 us, 3000^3 through the staged kernel 150 us).
-//
-// M and N.  Rule: fp32/fp16, k a whole number of ring slices, both m and n at least 512, at least 20 GFLOP (below
-// that the two extra launches cost more than the block gains: 2000 x 2000 x 512 measured twice as slow cut up), and
-// m or n not a multiple of 64 (otherwise a whole-tile kernel takes the whole problem anyway).  The block is cut at
-// multiples of 128 (64 below 1024).  Measured cut up against one staged launch: HGEMM 8200 x 8200 x 8192 1.70 x,
-// 3000 x 3000 x 3008 1.36 x, SGEMM 6000 x 520 x 4096 1.55 x, 5000 x 3000 x 2048 TN 1.28 x; never below 0.98 x.
-static bool auto_decomposition(int dtype, size_t m, size_t n, size_t k, int batch, size_t *m0, size_t *n0)
+// Large problems with a ragged M or N that the x16 kernel's edge tiles cannot take (x16_edge_ok: a memory-contiguous
+// dimension that is not a whole number of 16-byte groups, which needs a padded leading dimension to get this far):
+// the whole-tile kernels are 2-3 times faster than the staged kernel on the part they can take, so the problem is
+// cut into a block of whole groups and up to two strips of fewer than eight rows or columns, each C element written
+// by exactly one launch.  Rule: fp32/fp16, both m and n at least 512, at least 20 GFLOP (below that the extra
+// launches cost more than the block gains).
+static bool auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
+                               size_t *n0)
 {
     if (dtype != MMBO_F32 && dtype != MMBO_F16) return false;
-    if (k == 0 || k % (size_t)ring_bk(dtype) != 0) return false;
+    if (k == 0) return false;
     if (m < 512 || n < 512) return false;
-    if (m % 64 == 0 && n % 64 == 0) return false;
+    if (x16_edge_ok(dtype, transA, transB, m, n)) return false;
     if (2.0 * (double)m * (double)n * (double)k * (double)(batch > 0 ? batch : 1) < 2e10) return false;
-    const size_t t = (m < 1024 || n < 1024) ? 64 : 128;
-    *m0 = m / t * t;
-    *n0 = n / t * t;
-    return true;
-}
-
-// K.  A k that is not a whole number of ring slices keeps a large problem off the whole-tile kernels altogether.
-// Rule: same element types, m and n at least 2048, k at least 1024, at least 20 GFLOP: the last k % slice columns of A
-// and rows of B go through the staged kernel first (C1 = alpha*A_tail*B_tail + beta*C, one pass over C), the first
-// k0 through MMBO_CONFIG_AUTO again as C = alpha*A0*B0 + 1*C1.  C1 is stored in C's element type: an fp16 result
-// is then rounded twice (fp32: the extra rounding is below the accumulation error).  Measured against one staged
-// launch: HGEMM 7000^3 TN 1.65 x, 8192 x 8192 x 8200 1.16 x, 2048 x 2048 x 3000 1.11 x, 3000^3 1.04 x; SGEMM 4100^3 NT
-// 2.0 x, 3000^3 1.19 x (1024 x 1024 x 10000 would lose 10 %: below the size limit).  Tightly packed operands with a
-// ragged leading dimension (NN with ldb = k) are not 16-byte aligned per column and stay with the staged kernel.
-static bool auto_k_split(int dtype, size_t m, size_t n, size_t k, int batch, size_t *k0)
-{
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return false;
-    const size_t bk = (size_t)ring_bk(dtype);
-    if (k < 1024 || k % bk == 0) return false;
-    if (m < 2048 || n < 2048) return false;
-    if (2.0 * (double)m * (double)n * (double)k * (double)(batch > 0 ? batch : 1) < 2e10) return false;
-    *k0 = k / bk * bk;
+    const size_t per16 = dtype == MMBO_F32 ? 4 : 8;
+    *m0 = transA ? m : m / per16 * per16;
+    *n0 = transB ? n / per16 * per16 : n;
     return true;
 }
 
 int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                            size_t *n0, size_t *k0)
+                            size_t *n0)
 {
     if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
     if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
-    if (!m0 || !n0 || !k0) return -MMBO_ERR_NULL_POINTER;
+    if (!m0 || !n0) return -MMBO_ERR_NULL_POINTER;
     *m0 = m;
     *n0 = n;
-    *k0 = k;
-    const bool ks = auto_k_split(dtype, m, n, k, batch, k0);
-    const bool mn = auto_decomposition(dtype, m, n, *k0, batch, m0, n0);
-    return ks || mn ? 1 : 0;
+    return auto_decomposition(dtype, transA, transB, m, n, k, batch, m0, n0) ? 1 : 0;
 }
 
 int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
@@ -575,23 +573,11 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (config_id == MMBO_CONFIG_AUTO) {
         // A large problem with ragged M or N: a whole-tile block plus up to two edge strips, each C element written
         // by exactly one of the launches (A and B must qualify for the whole-tile kernels, or nothing is gained).
-        size_t m0 = 0, n0 = 0, k0 = 0;
+        size_t m0 = 0, n0 = 0;
         const bool whole_tile_operands = (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 && (lda * esz_in) % 16 == 0 &&
                                          (ldb * esz_in) % 16 == 0 && ((size_t)strideA * esz_in) % 16 == 0 &&
                                          ((size_t)strideB * esz_in) % 16 == 0;
-        if (whole_tile_operands && auto_k_split(dtype, m, n, k, batch, &k0)) {
-            // the K tail first, with the caller's beta; then the whole slices on top of it
-            const char *a8 = static_cast<const char *>(A), *b8 = static_cast<const char *>(B);
-            const size_t off_a = (transA ? k0 : k0 * lda) * esz_in, off_b = (transB ? k0 * ldb : k0) * esz_in;
-            int rc = mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k - k0, alpha, a8 + off_a, lda, strideA,
-                                               b8 + off_b, ldb, strideB, beta, C, ldc, strideC, batch,
-                                               select_staged(dtype, m, n, k - k0, batch), stream);
-            if (rc != MMBO_OK) return rc;
-            const float one = 1.0f;
-            return mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k0, alpha, A, lda, strideA, B, ldb, strideB, &one,
-                                             C, ldc, strideC, batch, MMBO_CONFIG_AUTO, stream);
-        }
-        if (whole_tile_operands && auto_decomposition(dtype, m, n, k, batch, &m0, &n0)) {
+        if (whole_tile_operands && auto_decomposition(dtype, transA, transB, m, n, k, batch, &m0, &n0)) {
             const char *a8 = static_cast<const char *>(A), *b8 = static_cast<const char *>(B);
             char *c8 = static_cast<char *>(C);
             int rc = mmbo_gemm_strided_batched(dtype, transA, transB, m0, n0, k, alpha, A, lda, strideA, B, ldb, strideB,
@@ -640,7 +626,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     int split = cref.split;
     const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
     TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0} : tile_row(dtype, cref.tile);
-    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
+    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, transA, transB, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
@@ -653,7 +639,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (stages < 1) stages = 1;
     if ((size_t)split > stages) split = (int)stages;
     size_t k_per_split = ceil_div(stages, (size_t)split) * r.bk;
-    split = (int)ceil_div(k ? k : 1, k_per_split);
+    if (cref.ring && split > 1) k_per_split = k / r.bk / split * r.bk;      // whole slices; the last split also takes a partial one
+    else split = (int)ceil_div(k ? k : 1, k_per_split);
     if ((size_t)batch * split > 65535) return MMBO_ERR_INVALID_SIZE;
 
     GemmArgs a;

@@ -16,8 +16,7 @@
  *     alpha and beta are HOST pointers read before the call returns (src/gemm/gemm.h:31-32);
  *   - MMBO_F32: float A, B, C, alpha, beta; fp32 MFMA accumulate.
  *     MMBO_F16: IEEE binary16 A, B, C; alpha and beta are float; fp32 MFMA accumulate,
- *     one round-to-nearest-even to binary16 on the store (two where MMBO_CONFIG_AUTO splits K:
- *     mmbo_auto_decomposition).
+ *     one round-to-nearest-even to binary16 on the store.
  *     MMBO_F64: double A, B, C, alpha, beta (the reference's own element type); fp64 MFMA accumulate;
  *   - the launch is asynchronous on `stream` (a hipStream_t, NULL = the null stream the
  *     reference uses, src/gemm/common.h:12); the caller synchronises.  Configs with GlobalSplitU > 1 keep their
@@ -101,18 +100,18 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out);
  * negative mmbo_status on bad arguments.  Pure host logic: needs no device. */
 int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch);
 
-/* What MMBO_CONFIG_AUTO does with a large problem that is not made of whole tiles (and whose A and B are 16-byte
- * aligned).  M, N: the block [0, m0) x [0, n0), cut at tile multiples, goes to a whole-tile kernel, the columns
- * n0 .. n and the rows m0 .. m of the first n0 columns go to the staged kernel in up to two further launches on the
- * same stream; every element of C is written by exactly one of them.  K: when k is not a whole number of the
- * whole-tile kernels' slices (32 for fp16, 16 for fp32), the last k - k0 go through the staged kernel first
- * (C1 = alpha*A_tail*B_tail + beta*C) and the first k0 are added on top (C = alpha*A0*B0 + C1); C1 is stored in C's
- * element type, so an MMBO_F16 result is rounded twice in that case.  Name a config id to get one launch and one
- * rounding.  Returns 1 and the cuts when a rule applies to the shape, 0 (and m0 = m, n0 = n, k0 = k) when the call
- * is a single launch, a negative mmbo_status on bad arguments.  The reference's kernels take whole tiles only
- * (src/gemm/ref/Kernels.cpp:153-1123 has no edge handling).  Pure host logic: needs no device. */
+/* What MMBO_CONFIG_AUTO does with a large problem whose ragged M or N the kernels' own edge tiles cannot take.
+ * The fast kernels handle edge tiles and a partial last slice of k themselves, provided that a dimension which is
+ * contiguous in memory -- m under transA = N, n under transB = T -- is a whole number of 16-byte groups (8 halves,
+ * 4 floats) and that A and B are 16-byte aligned.  Where only the first condition fails (which takes a padded
+ * leading dimension), a large problem is cut: the block [0, m0) x [0, n0) of whole groups goes to a fast kernel, the
+ * columns n0 .. n and the rows m0 .. m of the first n0 columns go to the general kernel in up to two further launches
+ * on the same stream; every element of C is written by exactly one of them, from the full k.  Returns 1 and the cuts
+ * when the rule applies to the shape, 0 (and m0 = m, n0 = n) when the call is a single launch, a negative
+ * mmbo_status on bad arguments.  The reference's kernels take whole tiles only (its launcher floors the grid,
+ * src/gemm/driver.h:49-50).  Pure host logic: needs no device. */
 int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                            size_t *n0, size_t *k0);
+                            size_t *n0);
 
 /* Host twin of the kernels' work-group -> tile mapping: linear work-group id to (tile row, tile
  * column).  With num_xcd = 1 and linear_id = wg0 + wg1*nwg0 this is the reference's

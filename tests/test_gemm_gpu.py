@@ -73,16 +73,27 @@ def test_cfg5_strided_batched_hgemm_tn():
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
 def test_every_config_every_transpose_ragged(dtype, ta, tb):
+    """257 x 131 x 1000 through every config id.  The general kernel takes it in every config.  Of the direct-to-LDS
+    kernels the ring family only takes whole tiles, and the x16 family takes this shape in TN alone (m and n odd: neither
+    may be contiguous in memory; lda = ldb = 1000 keeps the columns 16-byte aligned) and only with a split-K factor that
+    divides the whole slices of this k (31 for fp16, 62 for fp32): everything else must be refused, never computed wrongly."""
     import gemm_mmbo_amd as G
+    taken = 0
     for cid in range(G.num_configs(dtype)):
+        name = G.config_info(dtype, cid)["name"]
         p = U.Problem(dtype, ta, tb, 257, 131, 1000, 1.5, 0.5, lda=None, ldc=260, seed=10 + cid)
-        if "DTL1" in G.config_info(dtype, cid)["name"]:
-            # the direct-to-LDS kernel only takes whole 256 x 256 x 32 tiles: a ragged shape must be refused
+        if "DTL1" in name:
+            d = G.config_info(dtype, cid)
+            if "MFMA16x16" in name and ta and not tb and (1000 // d["depth_u"]) % d["split_k"] == 0:
+                _run_and_check(p, cid, label=f"config {cid} {name}")
+                taken += 1
+                continue
             with pytest.raises(G.MmboError) as e:
                 U.run_gpu(p, cid)
             assert e.value.status == 5
             continue
-        _run_and_check(p, cid, label=f"config {cid} {G.config_info(dtype, cid)['name']}")
+        _run_and_check(p, cid, label=f"config {cid} {name}")
+    assert taken == ((5 if dtype == F16 else 10) if ta and not tb else 0)       # five x16 tiles; fp32 also with GlobalSplitU 2
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -189,10 +200,47 @@ def test_x16_kernel_every_config_every_transpose(dtype, ta, tb):
     assert ran == 125
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
+    """Ragged problems in the x16 kernel, by explicit config id, every tile and split-K factor: m and n that end inside
+    a tile (loads repeat the last rows, stores are guarded: the reference's edge handling, src/gemm/ref/Kernels.cpp:
+    1007-1121), down to one 16-byte group and, where the dimension is not contiguous in memory, odd sizes; a k that ends
+    inside a slice (zero-filled: the reference's tail loop, :921-1005), down to k smaller than one slice; with beta,
+    batches, and padded leading dimensions whose padding rows of C must stay untouched."""
+    import gemm_mmbo_amd as G
+    bk = 16 if dtype == F32 else 32
+    g = 4 if dtype == F32 else 8                                # elements per 16 bytes
+    ran = 0
+    for cid in _x16_ids(dtype):
+        d = G.config_info(dtype, cid)
+        bm, bn, sp = d["macro_tile_m"], d["macro_tile_n"], d["split_k"]
+        #        m            n        slices alpha beta batch pad k tail
+        cases = [(bm + g, 2 * bn - g, 3, 1.0, 0.0, 1, 0, 0), (2 * bm - 3 * g, bn + 5 * g, 7, 1.5, 0.5, 2, 8, 0), (g, bn, 2, 1.0, 0.0, 1, 0, 0),
+                 (bm, bn, 2, 1.0, 0.0, 1, 0, 1), (bm + g, bn - g, 3, 1.5, 0.5, 2, 8, bk - 1), (2 * bm, bn, 0 if sp == 1 else 1, 1.0, 0.0, 1, 0, 5),
+                 (bm, 2 * bn, 6, -1.0, 1.0, 1, 0, g), (bm - g, bn + g, 11, 1.0, 0.0, 1, 8, bk // 2 + 1)]
+        if ta:
+            cases.append((bm + 3, bn + g, 5, -1.0, 1.0, 1, 0, 0))
+        if not tb:
+            cases.append((bm + g, bn - 1, 6, 1.0, 0.5, 1, 0, 3))
+        if ta and not tb:
+            cases.append((bm - 1, 2 * bn + 1, 4, 1.0, 0.0, 1, 8, 7))
+        for (m, n, slices, alpha, beta, batch, pad, kt) in cases:
+            k = bk * slices * sp + kt
+            ar, br = U.stored_shape(ta, m, k)[0], U.stored_shape(tb, k, n)[0]
+            lda, ldb = -(-ar // g) * g + pad, -(-br // g) * g + pad       # columns of A and B start on 16-byte boundaries
+            p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, lda=lda, ldb=ldb, ldc=m + (3 if pad else 0), batch=batch,
+                          seed=900 + cid + slices, dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
+            _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch}")
+            ran += 1
+    assert ran >= 25 * 8
+
+
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
-    ragged border of tiles, against the oracle.  Ragged shapes and unaligned operands are refused; ld > dim and the
-    automatic pick work."""
+    ragged border of tiles, against the oracle.  Shapes the edge tiles cannot take and unaligned operands are refused;
+    ld > dim and the automatic pick work."""
     import gemm_mmbo_amd as G
     ids = _x16_ids()
     for cid in ids[:2]:
@@ -201,9 +249,10 @@ def test_x16_kernel_chip_block_order_and_refusals():
             p = U.Problem(F16, 0, 0, m, n, k, 1.0, 0.0, seed=300 + m // 256, dist="normal", c_fill="nan")
             _run_and_check(p, cid, label=f"chip blocks {m}x{n}x{k}")
     cid = ids[0]
-    for (dtype, m, n, k, offs) in ((F16, 255, 256, 128, (0, 0, 0)), (F16, 256, 300, 128, (0, 0, 0)), (F16, 256, 256, 136, (0, 0, 0)),
-                                   (F16, 256, 256, 128, (1, 0, 0)), (F32, 256, 256, 136, (0, 0, 0))):
-        p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
+    # a contiguous m (transA = N) or n (transB = T) that is not a whole number of 16-byte groups, unaligned A
+    for (dtype, ta, tb, m, n, k, offs) in ((F16, 0, 0, 255, 256, 128, (0, 0, 0)), (F16, 0, 1, 256, 300, 128, (0, 0, 0)),
+                                           (F16, 0, 0, 256, 256, 128, (1, 0, 0)), (F32, 0, 0, 254, 256, 136, (0, 0, 0))):
+        p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
         with pytest.raises(G.MmboError) as e:
             U.run_gpu(p, cid, offs)
         assert e.value.status == 5
@@ -491,25 +540,31 @@ def test_automatic_pick_never_fails_on_its_own_choice():
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
-def test_large_ragged_problems_are_cut_into_block_and_strips(dtype):
-    """MMBO_CONFIG_AUTO on shapes mmbo_auto_decomposition applies to: a whole-tile block and up to two strips, every
-    element of C written once; against the oracle, with beta, ld > dim (padding rows untouched), every transpose, a
-    batch, and bit-identical on repetition."""
+def test_large_ragged_problems_through_the_automatic_pick(dtype):
+    """MMBO_CONFIG_AUTO on large shapes that are not made of whole tiles: one launch of the x16 kernel (edge tiles, a
+    zero-filled last slice of k) where a contiguous m or n is a whole number of 16-byte groups, a block and up to two thin
+    strips (mmbo_auto_decomposition) where it is not, the general kernel where A or B is not 16-byte aligned.  Against
+    the oracle, with beta, ld > dim (padding rows untouched), every transpose, batches, bit-identical on repetition."""
     import gemm_mmbo_amd as G
     dist = "normal" if dtype == F16 else "uniform"
     cases = [(0, 0, 2100, 2300, 2560, 1.0, 0.0, {}), (0, 1, 2100, 2048, 2560, -1.0, 1.0, {}), (1, 0, 2048, 2100, 2560, 1.5, 0.5, {}),
              (1, 1, 1500, 1900, 4096, 1.0, 0.0, {}), (0, 0, 2100, 2300, 2560, 1.0, 1.0, {"lda": 2104, "ldb": 2568, "ldc": 2111}),
              (0, 1, 1200, 1300, 2304, 1.0, 0.5, {"batch": 3}),
-             # K that is not a whole number of slices: a tail pass first, then the whole slices on top
+             (0, 1, 2306, 2101, 2560, 1.5, 0.5, {"lda": 2312, "ldb": 2104, "ldc": 2307}),
+             (0, 0, 2102, 2302, 2576, 1.0, 0.5, {"lda": 2104, "ldb": 2576}),
              (0, 0, 2104, 2304, 2568, 1.0, 0.0, {}), (1, 0, 2048, 2048, 3000, -1.0, 1.0, {}), (0, 1, 2048, 2304, 2570, 1.5, 0.5, {}),
-             (1, 1, 2056, 2048, 1208, 1.0, 0.5, {"batch": 2})]
+             (1, 1, 2056, 2048, 1208, 1.0, 0.5, {"batch": 2}), (1, 0, 2051, 2049, 2563, 1.0, 0.0, {"lda": 2568, "ldb": 2568})]
+    cut = 0
     for (ta, tb, m, n, k, alpha, beta, kw) in cases:
         batch = kw.get("batch", 1)
-        assert G.auto_decomposition(dtype, ta, tb, m, n, k, batch) is not None
+        cut += G.auto_decomposition(dtype, ta, tb, m, n, k, batch) is not None
         p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, seed=500 + m + n, dist=dist, c_fill="uniform" if beta else "nan", **kw)
-        got = _run_and_check(p, -1, label=f"decomposed {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} {kw}")
+        got = _run_and_check(p, -1, label=f"ragged {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} {kw}")
         again, _ = U.run_gpu(p, -1)
         assert np.array_equal(got.view(U.BITS[dtype]), again.view(U.BITS[dtype]))
-    # unaligned A: the rule's shape applies, the operands do not: one staged launch, same result bar
+    assert cut >= 2                                             # some of the cases above were cut up, most were not
+    assert G.auto_decomposition(dtype, 0, 1, 2306, 2101, 2560) == ((2304, 2100) if dtype == F32 else (2304, 2096))
+    assert G.auto_decomposition(dtype, 1, 0, 2051, 2049, 2563) is None
+    # unaligned A: one launch of the general kernel, same result bar
     p = U.Problem(dtype, 0, 0, 2100, 2300, 2560, 1.0, 0.0, seed=77, dist=dist, c_fill="nan")
     _run_and_check(p, -1, label="ragged, unaligned A", offsets=(1, 0, 0))
