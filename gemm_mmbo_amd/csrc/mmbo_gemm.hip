@@ -61,16 +61,15 @@ inline bool x16_edge_ok(int dtype, int transA, int transB, size_t m, size_t n)
 }
 
 // Does the ring (x16 = false) or x16 config (tile, split) take this shape?  Ring: m, n whole tiles, k whole slices, the
-// same number for every split.  x16: whole tiles or x16_edge_ok; every split gets the same number of whole slices
-// (at least one when there is more than one split) and the last split the partial slice, if any.
+// same number for every split.  x16: x16_edge_ok (whole tiles always are), any k; the splits take equal runs of whole slices and
+// the last one what is left, partial slice included (fewer splits than asked for when k is short).
 inline bool ring_shape_ok(int dtype, int tile, int split, int transA, int transB, size_t m, size_t n, size_t k, bool x16)
 {
     const RingRow &r = x16 ? kX16Tiles[tile] : kRingTiles[tile];
     const size_t bk = (size_t)ring_bk(dtype);
     if (k == 0) return false;
-    const bool ragged = m % r.bm || n % r.bn || k % bk;
-    if (ragged && !(x16 && x16_edge_ok(dtype, transA, transB, m, n))) return false;
-    if (split > 1 && k / bk < (size_t)split) return false;
+    if (x16) return x16_edge_ok(dtype, transA, transB, m, n);
+    if (m % r.bm || n % r.bn || k % bk) return false;
     return (k / bk) % (size_t)split == 0;
 }
 
@@ -361,7 +360,12 @@ static bool tile_span_ok(const TileRow &r, int transA, int transB, size_t lda, s
 // C traffic; the last, partial round runs with fewer work-groups per CU; split-K adds the reduction launch.  The
 // constants are a least-squares fit to the times of every such config on 45 shapes (gemm_mmbo_amd/tune.py --dump);
 // on those shapes the model's pick is within 2.5 % of the fastest config on average, 21 % at worst.
-static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, size_t n, size_t k, int batch)
+// split_lines: the rows of a packed operand (leading dimension = its stored row count) do not start on 128-byte lines,
+// so every request of the direct loads touches one line more.  Measured on fp16: the 128 x 128 and smaller tiles, which
+// are bound by that stream, lose 13-26 % of their in-loop rate (3000^3 against 3072^3, 4104^3 against 4096^3, 8200 against
+// 8192), the 256 x 256 tile up to 15 % at 3000 and nothing at 4104 or 8200; fp32 tiles, MFMA-bound, lose nothing.
+static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, size_t n, size_t k, int batch,
+                              bool split_lines = false)
 {
     static const double eff[2][2][NUM_RING_TILES] = {
         // 256x256 128x128 128x64  64x64
@@ -379,8 +383,9 @@ static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, 
     if (per_cu < 1) per_cu = 1;
     const double cus = 256.0;
     const double wgs = (double)ceil_div(m, (size_t)r.bm) * (double)ceil_div(n, (size_t)r.bn) * split * batch;
-    const double slices = std::ceil((double)k / bk) / split;
-    const double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
+    const double slices = std::ceil(std::ceil((double)k / bk) / split);
+    double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
+    if (split_lines && dtype == MMBO_F16) e *= rt == 0 ? 0.95 : 0.78;
     auto tile_time = [&](double resident) {
         return fill + slices * (2.0 * r.bm * r.bn * bk / flop_per_us_cu) * resident / e +
                c_us_per_kb * r.bm * r.bn * esz * resident / 1e3;
@@ -442,6 +447,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         static const int x16_of_ring[NUM_RING_TILES] = {0, 2, 3, 4};       // same macro tile in kX16Tiles (256 x 256: four wavefronts)
         int pick = -1;
         double pick_t = 0.0;
+        const size_t esz = dtype == MMBO_F32 ? 4 : 2;
+        const bool split_lines = ((transA ? k : m) * esz) % 128 != 0 || ((transB ? n : k) * esz) % 128 != 0;
         for (int rt = 0; rt < NUM_RING_TILES; ++rt)
             for (int si = 0; si < NUM_SPLITS; ++si) {
                 const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], transA, transB, m, n, k, false);
@@ -454,7 +461,7 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
                 bool x16 = dtype == MMBO_F16 ? rt != 3 : (rt == 0 && !(transA == 0 && transB == 1));
                 if (!ring_ok) x16 = true;           // ragged M or N: only the x16 kernel has edge tiles
                 if (!x16_ok) x16 = false;
-                const double t = model_time_ring(dtype, x16, rt, kSplits[si], m, n, k, batch);
+                const double t = model_time_ring(dtype, x16, rt, kSplits[si], m, n, k, batch, split_lines);
                 if (pick < 0 || t < pick_t) {
                     pick_t = t;
                     pick = x16 ? x16_config_id(x16_of_ring[rt], si) : ring_config_id(rt, si);
@@ -639,8 +646,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (stages < 1) stages = 1;
     if ((size_t)split > stages) split = (int)stages;
     size_t k_per_split = ceil_div(stages, (size_t)split) * r.bk;
-    if (cref.ring && split > 1) k_per_split = k / r.bk / split * r.bk;      // whole slices; the last split also takes a partial one
-    else split = (int)ceil_div(k ? k : 1, k_per_split);
+    split = (int)ceil_div(k ? k : 1, k_per_split);        // the last split takes what is left, a partial slice included
     if ((size_t)batch * split > 65535) return MMBO_ERR_INVALID_SIZE;
 
     GemmArgs a;

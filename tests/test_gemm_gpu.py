@@ -75,16 +75,15 @@ def test_cfg5_strided_batched_hgemm_tn():
 def test_every_config_every_transpose_ragged(dtype, ta, tb):
     """257 x 131 x 1000 through every config id.  The general kernel takes it in every config.  Of the direct-to-LDS
     kernels the ring family only takes whole tiles, and the x16 family takes this shape in TN alone (m and n odd: neither
-    may be contiguous in memory; lda = ldb = 1000 keeps the columns 16-byte aligned) and only with a split-K factor that
-    divides the whole slices of this k (31 for fp16, 62 for fp32): everything else must be refused, never computed wrongly."""
+    may be contiguous in memory; lda = ldb = 1000 keeps the columns 16-byte aligned), with every split-K factor (31 or 62
+    whole slices and a partial one: the splits are uneven): everything else must be refused, never computed wrongly."""
     import gemm_mmbo_amd as G
     taken = 0
     for cid in range(G.num_configs(dtype)):
         name = G.config_info(dtype, cid)["name"]
         p = U.Problem(dtype, ta, tb, 257, 131, 1000, 1.5, 0.5, lda=None, ldc=260, seed=10 + cid)
         if "DTL1" in name:
-            d = G.config_info(dtype, cid)
-            if "MFMA16x16" in name and ta and not tb and (1000 // d["depth_u"]) % d["split_k"] == 0:
+            if "MFMA16x16" in name and ta and not tb:
                 _run_and_check(p, cid, label=f"config {cid} {name}")
                 taken += 1
                 continue
@@ -93,7 +92,7 @@ def test_every_config_every_transpose_ragged(dtype, ta, tb):
             assert e.value.status == 5
             continue
         _run_and_check(p, cid, label=f"config {cid} {name}")
-    assert taken == ((5 if dtype == F16 else 10) if ta and not tb else 0)       # five x16 tiles; fp32 also with GlobalSplitU 2
+    assert taken == (25 if ta and not tb else 0)
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -220,6 +219,8 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
         cases = [(bm + g, 2 * bn - g, 3, 1.0, 0.0, 1, 0, 0), (2 * bm - 3 * g, bn + 5 * g, 7, 1.5, 0.5, 2, 8, 0), (g, bn, 2, 1.0, 0.0, 1, 0, 0),
                  (bm, bn, 2, 1.0, 0.0, 1, 0, 1), (bm + g, bn - g, 3, 1.5, 0.5, 2, 8, bk - 1), (2 * bm, bn, 0 if sp == 1 else 1, 1.0, 0.0, 1, 0, 5),
                  (bm, 2 * bn, 6, -1.0, 1.0, 1, 0, g), (bm - g, bn + g, 11, 1.0, 0.0, 1, 8, bk // 2 + 1)]
+        if sp > 1:              # uneven splits: the last one gets fewer slices, only the partial one, or the count shrinks
+            cases += [(bm, bn + g, 5, 1.0, 0.0, 1, 0, bk * (sp - 1) + 3), (bm + g, bn, 1, 1.5, 0.5, 1, 0, bk + 1), (bm, bn, 0, 1.0, 0.0, 1, 0, bk * 2 + 9)]
         if ta:
             cases.append((bm + 3, bn + g, 5, -1.0, 1.0, 1, 0, 0))
         if not tb:
