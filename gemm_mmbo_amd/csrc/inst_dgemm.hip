@@ -30,8 +30,7 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
         attr_set[dev].store(true, std::memory_order_release);
     }
     dim3 grid(args.nwg0 * args.nwg1, 1, args.batch);
-    hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
-    return hipGetLastError();
+    return launch_kernel(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
 }
 
 template <bool TA, bool TB>

@@ -47,8 +47,7 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
         if (gx > (unsigned)n) gx = (unsigned)n;
     }
     dim3 grid(gx, 1, args.batch * args.splits);
-    hipLaunchKernelGGL(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
-    return hipGetLastError();
+    return launch_kernel(kernel, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
 }
 }  // namespace
 

@@ -6,6 +6,15 @@
 
 namespace mmbo {
 
+// Launches kernel(args) and returns the status of that launch alone (hipGetLastError would also hand back an error
+// that an earlier, unrelated HIP call of this thread -- the caller's own, another library's -- left behind).
+template <typename Kernel>
+inline hipError_t launch_kernel(Kernel kernel, dim3 grid, dim3 block, unsigned lds_bytes, hipStream_t stream, const GemmArgs &args)
+{
+    void *kargs[] = {const_cast<GemmArgs *>(&args)};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, kargs, lds_bytes, stream);
+}
+
 // dtype: 0 = fp32, 1 = fp16.  Launches the staged kernel for tile row TILE with the given
 // transposes; grid = (nwg0*nwg1, 1, batch*splits).  Returns the launch's hipError_t.
 template <int DTYPE, int TILE>

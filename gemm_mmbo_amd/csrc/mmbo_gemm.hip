@@ -242,14 +242,11 @@ hipError_t launch_splitk_reduce(int dtype, const GemmArgs &args, hipStream_t str
     size_t mn = (size_t)args.m * args.n;
     const bool vec4 = args.m % 4 == 0;                   // a thread then owns four consecutive rows of one column
     dim3 grid((unsigned)ceil_div(vec4 ? mn / 4 : mn, 256), 1, args.batch);
-    if (dtype == MMBO_F32) {
-        if (vec4) hipLaunchKernelGGL((splitk_reduce_kernel<float, true>), grid, dim3(256), 0, stream, args);
-        else hipLaunchKernelGGL((splitk_reduce_kernel<float, false>), grid, dim3(256), 0, stream, args);
-    } else {
-        if (vec4) hipLaunchKernelGGL((splitk_reduce_kernel<half_t, true>), grid, dim3(256), 0, stream, args);
-        else hipLaunchKernelGGL((splitk_reduce_kernel<half_t, false>), grid, dim3(256), 0, stream, args);
-    }
-    return hipGetLastError();
+    if (dtype == MMBO_F32)
+        return vec4 ? launch_kernel(splitk_reduce_kernel<float, true>, grid, dim3(256), 0, stream, args)
+                    : launch_kernel(splitk_reduce_kernel<float, false>, grid, dim3(256), 0, stream, args);
+    return vec4 ? launch_kernel(splitk_reduce_kernel<half_t, true>, grid, dim3(256), 0, stream, args)
+                : launch_kernel(splitk_reduce_kernel<half_t, false>, grid, dim3(256), 0, stream, args);
 }
 
 }  // namespace mmbo

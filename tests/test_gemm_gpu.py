@@ -569,3 +569,50 @@ def test_large_ragged_problems_through_the_automatic_pick(dtype):
     # unaligned A: one launch of the general kernel, same result bar
     p = U.Problem(dtype, 0, 0, 2100, 2300, 2560, 1.0, 0.0, seed=77, dist=dist, c_fill="nan")
     _run_and_check(p, -1, label="ragged, unaligned A", offsets=(1, 0, 0))
+
+
+def test_random_shapes_paddings_and_configs_against_the_oracle():
+    """240 seeded random problems: both element types, every transpose, m, n, k from 1 up (a few thousand for some),
+    leading dimensions padded, tight or off 16-byte alignment, batches, alpha/beta variants, through MMBO_CONFIG_AUTO
+    or a random x16 config id.  A named config may refuse the problem (status 5); whatever runs must match the oracle
+    and leave the padding rows and the guard words behind C untouched."""
+    import random
+
+    import gemm_mmbo_amd as G
+    rnd = random.Random(20240607)
+    x16 = {dt: _x16_ids(dt) for dt in (F32, F16)}
+    ran = refused = 0
+    for it in range(240):
+        dt = rnd.choice((F32, F16))
+        ta, tb = rnd.randint(0, 1), rnd.randint(0, 1)
+        g = 4 if dt == F32 else 8
+        big = rnd.random() < 0.15
+        m, n = rnd.randint(1, 4400 if big else 700), rnd.randint(1, 4400 if big else 700)
+        k = rnd.randint(1, 80 if big else 1500)
+        if rnd.random() < 0.7:                                  # mostly shapes the x16 edge tiles can take
+            if not ta:
+                m = max(g, m // g * g)
+            if tb:
+                n = max(g, n // g * g)
+        batch = 1 if big else rnd.choice((1, 1, 1, 2, 3))
+        ar, br = U.stored_shape(ta, m, k)[0], U.stored_shape(tb, k, n)[0]
+        pad = rnd.choice((0, 0, g, 3 * g))
+        if rnd.random() < 0.85:
+            lda, ldb = -(-ar // g) * g + pad, -(-br // g) * g + pad
+        else:
+            lda, ldb = ar + rnd.randint(0, 3), br + rnd.randint(0, 3)
+        alpha, beta = rnd.choice((1.0, -1.0, 1.5)), rnd.choice((0.0, 0.0, 1.0, 0.5))
+        cfg = -1 if rnd.random() < 0.5 else rnd.choice(x16[dt])
+        p = U.Problem(dt, ta, tb, m, n, k, alpha, beta, lda=lda, ldb=ldb, ldc=m + rnd.choice((0, 0, 1, 5)), batch=batch,
+                      seed=1000 + it, dist="normal" if dt == F16 else "uniform", c_fill="uniform" if beta else "nan")
+        label = f"case {it}: {NAMES[dt]} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} ld {lda},{ldb},{p.ldc} b{batch} cfg {cfg}"
+        try:
+            got, guard = U.run_gpu(p, cfg)
+        except G.MmboError as e:
+            assert cfg >= 0 and e.status == 5, label
+            refused += 1
+            continue
+        U.check(p, got, label)
+        assert np.all(guard == 0), label
+        ran += 1
+    assert ran >= 150 and refused >= 10
