@@ -19,7 +19,6 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmmbo_gemm.so")
 
 EXPORTS = (
     "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
-    "mmbo_auto_decomposition",
     "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
@@ -144,20 +143,6 @@ def select_config(dtype, transA, transB, m, n, k, batch=1):
     if c < 0:
         _check(-c)
     return c
-
-
-def auto_decomposition(dtype, transA, transB, m, n, k, batch=1):
-    """(m0, n0) of the block MMBO_CONFIG_AUTO cuts out of a large problem whose ragged M or N the fast kernels' edge
-    tiles cannot take, or None when the call is a single launch."""
-    L = lib()
-    L.mmbo_auto_decomposition.argtypes = [ctypes.c_int] * 3 + [ctypes.c_size_t] * 3 + [ctypes.c_int] + \
-        [ctypes.POINTER(ctypes.c_size_t)] * 2
-    L.mmbo_auto_decomposition.restype = ctypes.c_int
-    m0, n0 = ctypes.c_size_t(0), ctypes.c_size_t(0)
-    r = L.mmbo_auto_decomposition(dtype, transA, transB, m, n, k, batch, ctypes.byref(m0), ctypes.byref(n0))
-    if r < 0:
-        _check(-r)
-    return (m0.value, n0.value) if r == 1 else None
 
 
 def wg_remap(linear_id, nwg0, nwg1, wgm=8, num_xcd=8):

@@ -133,9 +133,12 @@ struct Tile {
 
     // global byte offset (from the tile origin of this slice) of the chunk that lands in LDS slot (wave*LPW + i)*64 + lane.
     // `valid` = rows of the tile that exist in the operand (R, or fewer for the last tile of a ragged dimension): the
-    // slots of the rows past the edge are filled with a copy of the last row (KC) or the last 16-byte group of rows
-    // (RC: the host guarantees that the dimension is a whole number of such groups) -- they only feed accumulators
-    // that are never stored, and every address stays inside the operand.
+    // slots of the rows past the edge are filled with a copy of the last row (KC) or of the last 16-byte group that
+    // holds an existing row (RC) -- they only feed accumulators that are never stored.  KC addresses stay inside the
+    // operand.  An RC dimension that is not a whole number of groups makes the last group reach up to 14 bytes past
+    // the last existing row: in every stored column but the last that is the padding up to the (16-byte aligned) next
+    // column; in the last one it may lie behind the end of the operand, but inside the aligned 16 bytes, hence the
+    // page, that hold the last existing element -- it cannot fault, and what it reads is never used.
     __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld, uint32_t valid)
     {
         const uint32_t q = wave * LPW + i;
@@ -146,7 +149,7 @@ struct Tile {
         } else {
             uint32_t k = q * KPI + lane / CPR;
             uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-            return k * ld * ESZ + min(chunk, valid * ESZ / 16 - 1) * 16;
+            return k * ld * ESZ + min(chunk, (valid * ESZ + 15) / 16 - 1) * 16;
         }
     }
 
@@ -180,7 +183,7 @@ struct Tile {
             } else {
                 uint32_t k = q * KPI + lane / CPR;
                 uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-                if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + min(chunk, valid * ESZ / 16 - 1) * 16);
+                if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + min(chunk, (valid * ESZ + 15) / 16 - 1) * 16);
             }
             *reinterpret_cast<u32x4 *>(dst + q * 1024 + lane * 16) = v;
         }

@@ -51,24 +51,16 @@ inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_
     return dtype == MMBO_F16 && transA == transB && m % 256 == 0 && n % 256 == 0 && k % 64 == 0 && k >= 512;
 }
 
-// The x16 kernel takes ragged problems (its loads repeat the last rows of an edge tile, its edge tiles store under
-// guards, a partial last slice of k is zero-filled): only a dimension of op(A) or op(B) that is contiguous in memory
-// must be a whole number of 16-byte groups -- m under transA = N, n under transB = T.
-inline bool x16_edge_ok(int dtype, int transA, int transB, size_t m, size_t n)
-{
-    const size_t per16 = dtype == MMBO_F32 ? 4 : 8;
-    return (transA || m % per16 == 0) && (!transB || n % per16 == 0);
-}
-
 // Does the ring (x16 = false) or x16 config (tile, split) take this shape?  Ring: m, n whole tiles, k whole slices, the
-// same number for every split.  x16: x16_edge_ok (whole tiles always are), any k; the splits take equal runs of whole slices and
-// the last one what is left, partial slice included (fewer splits than asked for when k is short).
-inline bool ring_shape_ok(int dtype, int tile, int split, int transA, int transB, size_t m, size_t n, size_t k, bool x16)
+// same number for every split.  x16: any shape (its loads repeat the last rows of an edge tile, its edge tiles store
+// under guards, a partial last slice of k is zero-filled; the splits take equal runs of whole slices and the last one
+// what is left, fewer splits than asked for when k is short).  Both need 16-byte aligned A and B, checked at the call.
+inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k, bool x16)
 {
-    const RingRow &r = x16 ? kX16Tiles[tile] : kRingTiles[tile];
-    const size_t bk = (size_t)ring_bk(dtype);
     if (k == 0) return false;
-    if (x16) return x16_edge_ok(dtype, transA, transB, m, n);
+    if (x16) return true;
+    const RingRow &r = kRingTiles[tile];
+    const size_t bk = (size_t)ring_bk(dtype);
     if (m % r.bm || n % r.bn || k % bk) return false;
     return (k / bk) % (size_t)split == 0;
 }
@@ -448,8 +440,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         const bool split_lines = ((transA ? k : m) * esz) % 128 != 0 || ((transB ? n : k) * esz) % 128 != 0;
         for (int rt = 0; rt < NUM_RING_TILES; ++rt)
             for (int si = 0; si < NUM_SPLITS; ++si) {
-                const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], transA, transB, m, n, k, false);
-                const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], transA, transB, m, n, k, true);
+                const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], m, n, k, false);
+                const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], m, n, k, true);
                 if (!ring_ok && !x16_ok) continue;
                 // a dimension smaller than the tile stays with the staged kernel's smaller tiles
                 if (!ring_ok && (m < (size_t)kRingTiles[rt].bm || n < (size_t)kRingTiles[rt].bn)) continue;
@@ -467,37 +459,6 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         if (pick >= 0) return pick;
     }
     return select_staged(dtype, m, n, k, batch);
-}
-
-// Large problems with a ragged M or N that the x16 kernel's edge tiles cannot take (x16_edge_ok: a memory-contiguous
-// dimension that is not a whole number of 16-byte groups, which needs a padded leading dimension to get this far):
-// the whole-tile kernels are 2-3 times faster than the staged kernel on the part they can take, so the problem is
-// cut into a block of whole groups and up to two strips of fewer than eight rows or columns, each C element written
-// by exactly one launch.  Rule: fp32/fp16, both m and n at least 512, at least 20 GFLOP (below that the extra
-// launches cost more than the block gains).
-static bool auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                               size_t *n0)
-{
-    if (dtype != MMBO_F32 && dtype != MMBO_F16) return false;
-    if (k == 0) return false;
-    if (m < 512 || n < 512) return false;
-    if (x16_edge_ok(dtype, transA, transB, m, n)) return false;
-    if (2.0 * (double)m * (double)n * (double)k * (double)(batch > 0 ? batch : 1) < 2e10) return false;
-    const size_t per16 = dtype == MMBO_F32 ? 4 : 8;
-    *m0 = transA ? m : m / per16 * per16;
-    *n0 = transB ? n / per16 * per16 : n;
-    return true;
-}
-
-int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                            size_t *n0)
-{
-    if (!valid_dtype(dtype)) return -MMBO_ERR_INVALID_DTYPE;
-    if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
-    if (!m0 || !n0) return -MMBO_ERR_NULL_POINTER;
-    *m0 = m;
-    *n0 = n;
-    return auto_decomposition(dtype, transA, transB, m, n, k, batch, m0, n0) ? 1 : 0;
 }
 
 int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
@@ -575,33 +536,6 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
 
     const size_t esz_in = f64 ? 8 : dtype == MMBO_F32 ? 4 : 2;
     if (config_id == MMBO_CONFIG_AUTO) {
-        // A large problem with ragged M or N: a whole-tile block plus up to two edge strips, each C element written
-        // by exactly one of the launches (A and B must qualify for the whole-tile kernels, or nothing is gained).
-        size_t m0 = 0, n0 = 0;
-        const bool whole_tile_operands = (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 && (lda * esz_in) % 16 == 0 &&
-                                         (ldb * esz_in) % 16 == 0 && ((size_t)strideA * esz_in) % 16 == 0 &&
-                                         ((size_t)strideB * esz_in) % 16 == 0;
-        if (whole_tile_operands && auto_decomposition(dtype, transA, transB, m, n, k, batch, &m0, &n0)) {
-            const char *a8 = static_cast<const char *>(A), *b8 = static_cast<const char *>(B);
-            char *c8 = static_cast<char *>(C);
-            int rc = mmbo_gemm_strided_batched(dtype, transA, transB, m0, n0, k, alpha, A, lda, strideA, B, ldb, strideB,
-                                               beta, C, ldc, strideC, batch, MMBO_CONFIG_AUTO, stream);
-            if (rc != MMBO_OK) return rc;
-            if (n > n0) {           // right strip: all rows, columns n0 .. n
-                const size_t off_b = (transB ? n0 : n0 * ldb) * esz_in;
-                rc = mmbo_gemm_strided_batched(dtype, transA, transB, m, n - n0, k, alpha, A, lda, strideA, b8 + off_b, ldb,
-                                               strideB, beta, c8 + n0 * ldc * esz_in, ldc, strideC, batch, MMBO_CONFIG_AUTO,
-                                               stream);
-                if (rc != MMBO_OK) return rc;
-            }
-            if (m > m0) {           // bottom strip: rows m0 .. m of the first n0 columns
-                const size_t off_a = (transA ? m0 * lda : m0) * esz_in;
-                rc = mmbo_gemm_strided_batched(dtype, transA, transB, m - m0, n0, k, alpha, a8 + off_a, lda, strideA, B, ldb,
-                                               strideB, beta, c8 + m0 * esz_in, ldc, strideC, batch, MMBO_CONFIG_AUTO, stream);
-                if (rc != MMBO_OK) return rc;
-            }
-            return MMBO_OK;
-        }
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
         // The pick is made from the shape alone.  The whole-tile kernels also need 16-byte aligned A and B and a
@@ -630,7 +564,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     int split = cref.split;
     const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
     TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0} : tile_row(dtype, cref.tile);
-    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, transA, transB, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
+    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 

@@ -23,7 +23,15 @@
  *     partial sums in one workspace per device: two such GEMMs must not be in flight on different streams of
  *     one device at the same time (the same stream, or configs without split-K, are fine);
  *   - config_id selects a row of the tile-config table, like the reference's kernelId
- *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick;
+ *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick.  Every shape runs
+ *     under MMBO_CONFIG_AUTO.  Named configs: the general kernel's (no "DTL1" in the name) take any shape and
+ *     alignment; the direct-to-LDS ones ("DTL1") need A and B, their leading dimensions and batch strides 16-byte
+ *     aligned, and of those only the "MFMA16x16" family takes m, n that end inside a tile and k that ends inside a
+ *     slice (the reference's kernels take whole tiles only: its launcher floors the grid, src/gemm/driver.h:49-50).
+ *     That family fetches 16 bytes at a time: where m (transA = N) or n (transB = T) is not a whole number of such
+ *     groups, the fetch of the last group of a column covers up to 14 bytes behind its last element -- padding of
+ *     the leading dimension, or, for the very last column, bytes behind the matrix inside the aligned 16 bytes that
+ *     hold its last element; they are read and never used;
  *   - errors come back as status codes; nothing calls exit() (the reference's HIP_CHECK
  *     does, src/gemm/common.h:20-24).
  */
@@ -99,19 +107,6 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out);
  * src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:929-1177).  Returns a config id >= 0, or a
  * negative mmbo_status on bad arguments.  Pure host logic: needs no device. */
 int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch);
-
-/* What MMBO_CONFIG_AUTO does with a large problem whose ragged M or N the kernels' own edge tiles cannot take.
- * The fast kernels handle edge tiles and a partial last slice of k themselves, provided that a dimension which is
- * contiguous in memory -- m under transA = N, n under transB = T -- is a whole number of 16-byte groups (8 halves,
- * 4 floats) and that A and B are 16-byte aligned.  Where only the first condition fails (which takes a padded
- * leading dimension), a large problem is cut: the block [0, m0) x [0, n0) of whole groups goes to a fast kernel, the
- * columns n0 .. n and the rows m0 .. m of the first n0 columns go to the general kernel in up to two further launches
- * on the same stream; every element of C is written by exactly one of them, from the full k.  Returns 1 and the cuts
- * when the rule applies to the shape, 0 (and m0 = m, n0 = n) when the call is a single launch, a negative
- * mmbo_status on bad arguments.  The reference's kernels take whole tiles only (its launcher floors the grid,
- * src/gemm/driver.h:49-50).  Pure host logic: needs no device. */
-int mmbo_auto_decomposition(int dtype, int transA, int transB, size_t m, size_t n, size_t k, int batch, size_t *m0,
-                            size_t *n0);
 
 /* Host twin of the kernels' work-group -> tile mapping: linear work-group id to (tile row, tile
  * column).  With num_xcd = 1 and linear_id = wg0 + wg1*nwg0 this is the reference's

@@ -210,29 +210,17 @@ def test_tuner_shape_list_is_valid_and_rows_parse():
     # (the timing part needs the GPU: tests/test_gemm_gpu.py)
 
 
-def test_ragged_shapes_go_to_the_fast_kernels_or_are_cut():
-    """The x16 kernel takes ragged m, n and k as long as a memory-contiguous m or n is a whole number of 16-byte groups;
-    large problems that fail only that are cut into a block of whole groups and thin strips; small ones stay with the
-    general kernel."""
+def test_ragged_shapes_go_to_the_fast_kernels():
+    """The x16 kernel takes ragged m, n and k; only a dimension smaller than the smallest fast tile keeps a shape with the
+    general kernel (unaligned operands do too, but that is decided at the call, not from the shape)."""
     def name(dtype, ta, tb, m, n, k):
         return G.config_info(dtype, G.select_config(dtype, ta, tb, m, n, k))["name"]
-    assert G.auto_decomposition(G.F16, 0, 0, 3000, 3000, 3000) is None              # edge tiles and the k tail: the kernel's own
     assert "MFMA16x16" in name(G.F16, 0, 0, 3000, 3000, 3000)
     assert "MFMA16x16" in name(G.F32, 0, 1, 4100, 4100, 4099)
-    assert "MFMA16x16" in name(G.F16, 1, 0, 3001, 3003, 3005)                      # TN: neither m nor n is contiguous
-    assert G.auto_decomposition(G.F16, 1, 0, 3001, 3003, 3005) is None
-    assert G.auto_decomposition(G.F16, 0, 0, 3001, 3000, 3008) == (3000, 3000)      # m contiguous, 3001 halves: not whole groups
-    assert G.auto_decomposition(G.F32, 0, 1, 3001, 3002, 3000) == (3000, 3000)      # groups of four floats
-    assert G.auto_decomposition(G.F16, 0, 1, 4096, 4100, 4096) == (4096, 4096)      # only N ragged
-    assert "DTL1" not in name(G.F16, 0, 0, 3001, 3000, 3008)                       # the whole problem by name: general kernel
-    assert G.auto_decomposition(G.F16, 0, 0, 4096, 4096, 4096) is None              # whole tiles
-    assert G.auto_decomposition(G.F16, 0, 0, 1023, 777, 512) is None                # too little work
-    assert G.auto_decomposition(G.F16, 0, 0, 2001, 2000, 512) is None
-    assert G.auto_decomposition(G.F16, 0, 0, 401, 50000, 4096) is None              # a skinny side
-    assert G.auto_decomposition(G.F64, 0, 1, 3001, 3000, 3008) is None              # fp64: one kernel with edge handling
+    assert "MFMA16x16" in name(G.F16, 1, 0, 3001, 3003, 3005)
+    assert "MFMA16x16" in name(G.F16, 0, 0, 3001, 3000, 3008)
+    assert "MFMA16x16" in name(G.F32, 0, 1, 1001, 1002, 1000)
     assert "DTL1" not in name(G.F16, 0, 0, 8, 4096, 4096)                          # a dimension below the smallest fast tile
     assert "DTL1" in name(G.F16, 0, 0, 72, 4096, 4096)
-    for (m, n, k) in ((3001, 3000, 3008), (1001, 4100, 4096)):
-        m0, n0 = G.auto_decomposition(G.F16, 0, 0, m, n, k)
-        assert m0 % 8 == 0 and m - m0 < 8 and n0 == n
-        assert "MFMA16x16" in name(G.F16, 0, 0, m0, n0, k)
+    # large ragged shapes whose packed rows split cache lines: the 256 x 256 tile, not the bandwidth-bound smaller ones
+    assert G.config_info(G.F16, G.select_config(G.F16, 1, 0, 7000, 7000, 7008))["macro_tile_m"] == 256

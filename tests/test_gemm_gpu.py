@@ -205,7 +205,7 @@ def test_x16_kernel_every_config_every_transpose(dtype, ta, tb):
 def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
     """Ragged problems in the x16 kernel, by explicit config id, every tile and split-K factor: m and n that end inside
     a tile (loads repeat the last rows, stores are guarded: the reference's edge handling, src/gemm/ref/Kernels.cpp:
-    1007-1121), down to one 16-byte group and, where the dimension is not contiguous in memory, odd sizes; a k that ends
+    1007-1121), down to a single row or column, odd sizes also where the dimension is the contiguous one; a k that ends
     inside a slice (zero-filled: the reference's tail loop, :921-1005), down to k smaller than one slice; with beta,
     batches, and padded leading dimensions whose padding rows of C must stay untouched."""
     import gemm_mmbo_amd as G
@@ -221,12 +221,9 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
                  (bm, 2 * bn, 6, -1.0, 1.0, 1, 0, g), (bm - g, bn + g, 11, 1.0, 0.0, 1, 8, bk // 2 + 1)]
         if sp > 1:              # uneven splits: the last one gets fewer slices, only the partial one, or the count shrinks
             cases += [(bm, bn + g, 5, 1.0, 0.0, 1, 0, bk * (sp - 1) + 3), (bm + g, bn, 1, 1.5, 0.5, 1, 0, bk + 1), (bm, bn, 0, 1.0, 0.0, 1, 0, bk * 2 + 9)]
-        if ta:
-            cases.append((bm + 3, bn + g, 5, -1.0, 1.0, 1, 0, 0))
-        if not tb:
-            cases.append((bm + g, bn - 1, 6, 1.0, 0.5, 1, 0, 3))
-        if ta and not tb:
-            cases.append((bm - 1, 2 * bn + 1, 4, 1.0, 0.0, 1, 8, 7))
+        # m, n that end inside a 16-byte group (also where that dimension is the contiguous one) and inside a 4-row group
+        cases += [(bm + 3, bn + g, 5, -1.0, 1.0, 1, 0, 0), (bm + g, bn - 1, 6, 1.0, 0.5, 1, 0, 3), (bm - 1, 2 * bn + 1, 4, 1.0, 0.0, 2, 8, 7),
+                  (1, 1, 1, 1.0, 0.0, 1, 0, 1), (bm + g + 1, 3, 2, 1.5, 0.5, 1, 8, 0)]
         for (m, n, slices, alpha, beta, batch, pad, kt) in cases:
             k = bk * slices * sp + kt
             ar, br = U.stored_shape(ta, m, k)[0], U.stored_shape(tb, k, n)[0]
@@ -235,13 +232,12 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
                           seed=900 + cid + slices, dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
             _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch}")
             ran += 1
-    assert ran >= 25 * 8
+    assert ran >= 25 * 13
 
 
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
-    ragged border of tiles, against the oracle.  Shapes the edge tiles cannot take and unaligned operands are refused;
-    ld > dim and the automatic pick work."""
+    ragged border of tiles, against the oracle.  Unaligned operands are refused; ld > dim and the automatic pick work."""
     import gemm_mmbo_amd as G
     ids = _x16_ids()
     for cid in ids[:2]:
@@ -250,9 +246,9 @@ def test_x16_kernel_chip_block_order_and_refusals():
             p = U.Problem(F16, 0, 0, m, n, k, 1.0, 0.0, seed=300 + m // 256, dist="normal", c_fill="nan")
             _run_and_check(p, cid, label=f"chip blocks {m}x{n}x{k}")
     cid = ids[0]
-    # a contiguous m (transA = N) or n (transB = T) that is not a whole number of 16-byte groups, unaligned A
-    for (dtype, ta, tb, m, n, k, offs) in ((F16, 0, 0, 255, 256, 128, (0, 0, 0)), (F16, 0, 1, 256, 300, 128, (0, 0, 0)),
-                                           (F16, 0, 0, 256, 256, 128, (1, 0, 0)), (F32, 0, 0, 254, 256, 136, (0, 0, 0))):
+    # unaligned A or B (an element offset, a leading dimension that is not a whole number of 16-byte groups)
+    for (dtype, ta, tb, m, n, k, offs) in ((F16, 0, 0, 256, 256, 128, (1, 0, 0)), (F16, 0, 0, 256, 256, 128, (0, 4, 0)),
+                                           (F16, 0, 0, 255, 256, 128, (0, 0, 0)), (F32, 0, 1, 256, 254, 136, (0, 0, 0))):
         p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
         with pytest.raises(G.MmboError) as e:
             U.run_gpu(p, cid, offs)
@@ -543,9 +539,9 @@ def test_automatic_pick_never_fails_on_its_own_choice():
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_large_ragged_problems_through_the_automatic_pick(dtype):
     """MMBO_CONFIG_AUTO on large shapes that are not made of whole tiles: one launch of the x16 kernel (edge tiles, a
-    zero-filled last slice of k) where a contiguous m or n is a whole number of 16-byte groups, a block and up to two thin
-    strips (mmbo_auto_decomposition) where it is not, the general kernel where A or B is not 16-byte aligned.  Against
-    the oracle, with beta, ld > dim (padding rows untouched), every transpose, batches, bit-identical on repetition."""
+    zero-filled last slice of k, contiguous dimensions that end inside a 16-byte group), the general kernel where A or
+    B is not 16-byte aligned.  Against the oracle, with beta, ld > dim (padding rows untouched), every transpose, batches,
+    bit-identical on repetition."""
     import gemm_mmbo_amd as G
     dist = "normal" if dtype == F16 else "uniform"
     cases = [(0, 0, 2100, 2300, 2560, 1.0, 0.0, {}), (0, 1, 2100, 2048, 2560, -1.0, 1.0, {}), (1, 0, 2048, 2100, 2560, 1.5, 0.5, {}),
@@ -555,17 +551,11 @@ def test_large_ragged_problems_through_the_automatic_pick(dtype):
              (0, 0, 2102, 2302, 2576, 1.0, 0.5, {"lda": 2104, "ldb": 2576}),
              (0, 0, 2104, 2304, 2568, 1.0, 0.0, {}), (1, 0, 2048, 2048, 3000, -1.0, 1.0, {}), (0, 1, 2048, 2304, 2570, 1.5, 0.5, {}),
              (1, 1, 2056, 2048, 1208, 1.0, 0.5, {"batch": 2}), (1, 0, 2051, 2049, 2563, 1.0, 0.0, {"lda": 2568, "ldb": 2568})]
-    cut = 0
     for (ta, tb, m, n, k, alpha, beta, kw) in cases:
-        batch = kw.get("batch", 1)
-        cut += G.auto_decomposition(dtype, ta, tb, m, n, k, batch) is not None
         p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, seed=500 + m + n, dist=dist, c_fill="uniform" if beta else "nan", **kw)
         got = _run_and_check(p, -1, label=f"ragged {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} {kw}")
         again, _ = U.run_gpu(p, -1)
         assert np.array_equal(got.view(U.BITS[dtype]), again.view(U.BITS[dtype]))
-    assert cut >= 2                                             # some of the cases above were cut up, most were not
-    assert G.auto_decomposition(dtype, 0, 1, 2306, 2101, 2560) == ((2304, 2100) if dtype == F32 else (2304, 2096))
-    assert G.auto_decomposition(dtype, 1, 0, 2051, 2049, 2563) is None
     # unaligned A: one launch of the general kernel, same result bar
     p = U.Problem(dtype, 0, 0, 2100, 2300, 2560, 1.0, 0.0, seed=77, dist=dist, c_fill="nan")
     _run_and_check(p, -1, label="ragged, unaligned A", offsets=(1, 0, 0))
@@ -589,11 +579,6 @@ def test_random_shapes_paddings_and_configs_against_the_oracle():
         big = rnd.random() < 0.15
         m, n = rnd.randint(1, 4400 if big else 700), rnd.randint(1, 4400 if big else 700)
         k = rnd.randint(1, 80 if big else 1500)
-        if rnd.random() < 0.7:                                  # mostly shapes the x16 edge tiles can take
-            if not ta:
-                m = max(g, m // g * g)
-            if tb:
-                n = max(g, n // g * g)
         batch = 1 if big else rnd.choice((1, 1, 1, 2, 3))
         ar, br = U.stored_shape(ta, m, k)[0], U.stored_shape(tb, k, n)[0]
         pad = rnd.choice((0, 0, g, 3 * g))
