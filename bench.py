@@ -1,5 +1,5 @@
 """Headline benchmark: GEMM TFLOP/s at 8192^3 on one MI355X, fp16 (value) and fp32 (in "also"); "also" further
-carries the two HBM-bound skinny shapes (achieved algorithmic GB/s), the reference's own workload, DGEMM NT
+carries the two HBM-bound skinny shapes (achieved algorithmic GB/s), three ragged shapes, the reference's own workload, DGEMM NT
 44160 x 2048 x 384 with alpha = -1, beta = 1, and DGEMM at 8192^3.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
@@ -162,6 +162,43 @@ def skinny_legs(G, torch, steps, warmup):
     return out
 
 
+def ragged_legs(G, torch, steps, warmup):
+    """Shapes that end inside a tile and inside a slice of k (alpha = 1, beta = 0, tightly packed operands), one launch
+    each through the automatic pick: time per GEMM from events on the launch stream, TFLOP/s against the matrix peak.
+    Parity of ragged shapes is in tests/test_gemm_gpu.py."""
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(98)
+    out = {}
+    for dname, dtype, tdt, ta, tb, m, n, k in (("fp16", G.F16, torch.float16, 0, 0, 3000, 3000, 3000),
+                                               ("fp16", G.F16, torch.float16, 1, 0, 8192, 8192, 8200),
+                                               ("fp32", G.F32, torch.float32, 0, 1, 4100, 4100, 4096)):
+        A = (torch.rand(m * k, device="cuda", generator=gen) * 2 - 1).to(tdt)
+        B = (torch.rand(k * n, device="cuda", generator=gen) * 2 - 1).to(tdt)
+        C = torch.empty(m * n, device="cuda", dtype=tdt)
+        lda, ldb = (k if ta else m), (n if tb else k)
+        cid = G.select_config(dtype, ta, tb, m, n, k, 1)
+
+        def run():
+            G.gemm(dtype, ta, tb, m, n, k, 1.0, A, lda, B, ldb, 0.0, C, m, G.CONFIG_AUTO, stream)
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            run()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1e3
+        tf = 2.0 * m * n * k / us * 1e-6
+        out[f"{dname}_{'NT'[ta]}{'NT'[tb]}_{m}x{n}x{k}"] = {"us": round(us, 1), "tflops": round(tf, 1),
+                                                            "frac_of_peak": round(tf / PEAK_TFLOPS["f16" if dtype == G.F16 else "f32"], 4),
+                                                            "tile_config": G.config_info(dtype, cid)["name"]}
+        del A, B, C
+    return out
+
+
 def cpu_baseline(dtype, m, n, k, hA, hB):
     """The oracle's native-precision CPU GEMM (fp16 operands widened to fp32, fp32 multiply-add chains) on
     the same operands, all host cores, whole problem once."""
@@ -239,6 +276,7 @@ def main():
 
     f64 = dgemm_legs(G, torch, args.steps, args.warmup) if args.only in (None, "f64") else {}
     skinny = skinny_legs(G, torch, args.steps, args.warmup) if not args.only else {}
+    ragged = ragged_legs(G, torch, min(args.steps, 10), min(args.warmup, 3)) if not args.only else {}
     if args.only == "f64":
         print(json.dumps({"metric": METRIC, "also": f64}))
         return
@@ -286,6 +324,8 @@ def main():
         out["also"]["fp16_constant_operands_frac_of_peak"] = round(ones_tflops / PEAK_TFLOPS["f16"], 4)
     if skinny:
         out.setdefault("also", {})["skinny_nn_hbm_bound"] = skinny
+    if ragged:
+        out.setdefault("also", {})["ragged_one_launch"] = ragged
     if f64:
         out.setdefault("also", {}).update(f64)
         out["parity_ok"] = bool(out["parity_ok"] and f64["fp64_hpl_max_rel_err"] <= f64["fp64_hpl_rel_err_limit"]
