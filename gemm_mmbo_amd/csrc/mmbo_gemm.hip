@@ -443,8 +443,12 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
                 const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], m, n, k, false);
                 const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], m, n, k, true);
                 if (!ring_ok && !x16_ok) continue;
-                // a dimension smaller than the tile stays with the staged kernel's smaller tiles
-                if (!ring_ok && (m < (size_t)kRingTiles[rt].bm || n < (size_t)kRingTiles[rt].bn)) continue;
+                // A dimension smaller than the tile: only the 64 x 64 fp16 tile on a long k is worth it (measured against
+                // the staged kernel's 32 x 32 tile: HGEMM 16 x 4096 x 4096 11.8 against 17.5 us, 48 x 48 x 8192 10.1
+                // against 17.1, 32 x 8192 x 1024 9.1 against 8.5-9.4; SGEMM 4096 x 32 x 4096 27.4 against 22.9).
+                if (!ring_ok && (m < (size_t)kRingTiles[rt].bm || n < (size_t)kRingTiles[rt].bn) &&
+                    !(dtype == MMBO_F16 && rt == 3 && k >= 1024))
+                    continue;
                 if (kSplits[si] > 1 && (k / ring_bk(dtype)) / (size_t)kSplits[si] < 2) continue;      // slices too thin
                 if ((size_t)batch * kSplits[si] > 65535) continue;
                 bool x16 = dtype == MMBO_F16 ? rt != 3 : (rt == 0 && !(transA == 0 && transB == 1));

@@ -211,8 +211,8 @@ def test_tuner_shape_list_is_valid_and_rows_parse():
 
 
 def test_ragged_shapes_go_to_the_fast_kernels():
-    """The x16 kernel takes ragged m, n and k; only a dimension smaller than the smallest fast tile keeps a shape with the
-    general kernel (unaligned operands do too, but that is decided at the call, not from the shape)."""
+    """The x16 kernel takes ragged m, n and k; a dimension smaller than the smallest fast tile mostly keeps a shape with
+    the general kernel (unaligned operands do too, but that is decided at the call, not from the shape)."""
     def name(dtype, ta, tb, m, n, k):
         return G.config_info(dtype, G.select_config(dtype, ta, tb, m, n, k))["name"]
     assert "MFMA16x16" in name(G.F16, 0, 0, 3000, 3000, 3000)
@@ -220,7 +220,9 @@ def test_ragged_shapes_go_to_the_fast_kernels():
     assert "MFMA16x16" in name(G.F16, 1, 0, 3001, 3003, 3005)
     assert "MFMA16x16" in name(G.F16, 0, 0, 3001, 3000, 3008)
     assert "MFMA16x16" in name(G.F32, 0, 1, 1001, 1002, 1000)
-    assert "DTL1" not in name(G.F16, 0, 0, 8, 4096, 4096)                          # a dimension below the smallest fast tile
+    assert "DTL1" not in name(G.F32, 0, 0, 8, 4096, 4096)                          # a dimension below the smallest fast tile:
+    assert "DTL1" not in name(G.F16, 0, 0, 40, 40, 64)                             # general kernel, except fp16 on a long k
+    assert "MT064x064" in name(G.F16, 0, 0, 8, 4096, 4096) and "DTL1" in name(G.F16, 0, 0, 8, 4096, 4096)
     assert "DTL1" in name(G.F16, 0, 0, 72, 4096, 4096)
     # large ragged shapes whose packed rows split cache lines: the 256 x 256 tile, not the bandwidth-bound smaller ones
     assert G.config_info(G.F16, G.select_config(G.F16, 1, 0, 7000, 7000, 7008))["macro_tile_m"] == 256
