@@ -131,15 +131,24 @@ struct Tile {
     __device__ static inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ kc_swz(row)) << 4); }
     __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4); }
 
+    static constexpr uint32_t EPC = 16 / ESZ;                   // elements per 16-byte group
+
+    // RC operand, edge tile.  `valid` = rows of the tile that exist (R, or fewer for the last tile of a ragged
+    // dimension).  Groups before the last one that holds an existing row are fetched in place.  That last group is
+    // fetched from the 16 bytes that END at the last existing row (the reference's ShiftPtr, src/gemm/ref/Kernels.cpp:
+    // 240-304: no byte outside the operand is touched), so its slot holds rows valid-EPC .. valid-1 instead of
+    // last*EPC .. : the epilogue undoes the shift.  The slots of the groups behind it get the same 16 bytes and feed
+    // accumulators that are never stored.  A tile with fewer than EPC rows reaches back into the tile before it: the
+    // caller moves the tile origin back by `back` = EPC - valid rows (the host refuses a whole dimension that short).
+    __device__ static inline uint32_t rc_group_off(uint32_t chunk, uint32_t valid, uint32_t back)
+    {
+        const uint32_t last = (valid - 1) / EPC;
+        return chunk < last ? chunk * 16 : (valid + back - EPC) * ESZ;
+    }
+
     // global byte offset (from the tile origin of this slice) of the chunk that lands in LDS slot (wave*LPW + i)*64 + lane.
-    // `valid` = rows of the tile that exist in the operand (R, or fewer for the last tile of a ragged dimension): the
-    // slots of the rows past the edge are filled with a copy of the last row (KC) or of the last 16-byte group that
-    // holds an existing row (RC) -- they only feed accumulators that are never stored.  KC addresses stay inside the
-    // operand.  An RC dimension that is not a whole number of groups makes the last group reach up to 14 bytes past
-    // the last existing row: in every stored column but the last that is the padding up to the (16-byte aligned) next
-    // column; in the last one it may lie behind the end of the operand, but inside the aligned 16 bytes, hence the
-    // page, that hold the last existing element -- it cannot fault, and what it reads is never used.
-    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld, uint32_t valid)
+    // KC operand, edge tile: the slots of the rows past the edge are filled with a copy of the last existing row.
+    __device__ static inline uint32_t load_goff(int wave, int lane, int i, uint32_t ld, uint32_t valid, uint32_t back)
     {
         const uint32_t q = wave * LPW + i;
         if constexpr (KC) {
@@ -149,7 +158,7 @@ struct Tile {
         } else {
             uint32_t k = q * KPI + lane / CPR;
             uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-            return k * ld * ESZ + min(chunk, (valid * ESZ + 15) / 16 - 1) * 16;
+            return k * ld * ESZ + rc_group_off(chunk, valid, back);
         }
     }
 
@@ -157,10 +166,9 @@ struct Tile {
     // src/gemm/ref/Kernels.cpp:921-1005, zero-fills k >= remainder): the same slots as the direct loads fill, written
     // through registers, with zeros from k_tail on.  g = operand origin of this tile at the tail slice.  Only elements
     // that exist are read: a 16-byte chunk along k that straddles the end goes element by element.
-    __device__ static inline void fill_tail(const char *g, uint32_t ld, uint32_t valid, uint32_t k_tail, char *dst, int wave,
-                                            int lane)
+    __device__ static inline void fill_tail(const char *g, uint32_t ld, uint32_t valid, uint32_t back, uint32_t k_tail, char *dst,
+                                            int wave, int lane)
     {
-        constexpr uint32_t EPC = 16 / ESZ;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
             const uint32_t q = wave * LPW + i;
@@ -183,7 +191,7 @@ struct Tile {
             } else {
                 uint32_t k = q * KPI + lane / CPR;
                 uint32_t chunk = (lane % CPR) ^ rc_mask(k);
-                if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + min(chunk, (valid * ESZ + 15) / 16 - 1) * 16);
+                if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + rc_group_off(chunk, valid, back));
             }
             *reinterpret_cast<u32x4 *>(dst + q * 1024 + lane * 16) = v;
         }
@@ -324,22 +332,25 @@ gemm_x16_kernel(const GemmArgs args)
     const int n_slice = k_end > k_begin ? (int)((k_end - k_begin) / BK) : 0;
     const uint32_t k_tail = k_end > k_begin ? (k_end - k_begin) % BK : 0;
 
+    // rows and columns of this tile that exist: less than the tile on the last tile row / column of a ragged problem;
+    // a row-contiguous operand with less than one 16-byte group of them starts that many rows early (Tile::rc_group_off)
+    const uint32_t m_here = min((uint32_t)BM, args.m - row0), n_here = min((uint32_t)BN, args.n - col0);
+    constexpr uint32_t EPC = 16 / ESZ;
+    const uint32_t backA = (!TA && m_here < EPC) ? EPC - m_here : 0, backB = (TB && n_here < EPC) ? EPC - n_here : 0;
     const char *gA = static_cast<const char *>(args.A) +
                      ((int64_t)batch * args.strideA + (TA ? (int64_t)row0 * lda + k_begin
-                                                          : (int64_t)k_begin * lda + row0)) * ESZ;
+                                                          : (int64_t)k_begin * lda + row0 - backA)) * ESZ;
     const char *gB = static_cast<const char *>(args.B) +
-                     ((int64_t)batch * args.strideB + (TB ? (int64_t)k_begin * ldb + col0
+                     ((int64_t)batch * args.strideB + (TB ? (int64_t)k_begin * ldb + col0 - backB
                                                           : (int64_t)col0 * ldb + k_begin)) * ESZ;
     const int64_t stepA = (TA ? (int64_t)BK : (int64_t)BK * lda) * ESZ;
     const int64_t stepB = (TB ? (int64_t)BK * ldb : (int64_t)BK) * ESZ;
 
-    // rows and columns of this tile that exist: less than the tile on the last tile row / column of a ragged problem
-    const uint32_t m_here = min((uint32_t)BM, args.m - row0), n_here = min((uint32_t)BN, args.n - col0);
     uint32_t offA[TileA::LPW], offB[TileB::LPW];
 #pragma unroll
-    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda, m_here);
+    for (int i = 0; i < TileA::LPW; ++i) offA[i] = TileA::load_goff(wave, lane, i, lda, m_here, backA);
 #pragma unroll
-    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here);
+    for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here, backB);
 
     // direct load number l (A's first, then B's) of slice s into ring buffer `buf`
     auto issue_load = [&](auto L, const char *pa, const char *pb, char *dst) {
@@ -616,8 +627,8 @@ gemm_x16_kernel(const GemmArgs args)
     if (k_tail != 0) {
         // The partial last slice.  The loop ended on a barrier after every wavefront's last LDS read and with no load in
         // flight, so buffer 0 is free: fill it through registers (zeros from k_tail on), then one more slice of MFMAs.
-        TileA::fill_tail(gA + (int64_t)n_slice * stepA, lda, m_here, k_tail, lds, wave, lane);
-        TileB::fill_tail(gB + (int64_t)n_slice * stepB, ldb, n_here, k_tail, lds + TileA::BYTES, wave, lane);
+        TileA::fill_tail(gA + (int64_t)n_slice * stepA, lda, m_here, backA, k_tail, lds, wave, lane);
+        TileB::fill_tail(gB + (int64_t)n_slice * stepB, ldb, n_here, backB, k_tail, lds + TileA::BYTES, wave, lane);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         fa[0].read_all(lds_base, adA);
@@ -646,49 +657,67 @@ gemm_x16_kernel(const GemmArgs args)
     // workspace [split][batch][n][m] and the reduction kernel applies alpha and beta.
     const uint32_t wrow0 = row0 + wm * Cfg::TM + 4 * (lane >> 4), wcol0 = col0 + wn * Cfg::TN + (lane & 15);
     if (m_here < (uint32_t)BM || n_here < (uint32_t)BN) {
-        // Edge tile (reference: the guarded store, src/gemm/ref/Kernels.cpp:1064-1121): every element is tested against
-        // m and n; four rows go out as one vector where all four exist and C allows it.
+        // Edge tile (reference: the un-shift and the guarded store, src/gemm/ref/Kernels.cpp:1007-1121).  Tile row r is
+        // row r of C, except in the last 16-byte group of a row-contiguous A (Tile::rc_group_off): there tile rows
+        // gsm+shm .. gsm+EPC-1 are rows gsm .. m_here-1, and tile rows gsm .. gsm+shm-1 repeat rows that the group
+        // before already produced.  Columns likewise under a row-contiguous B.  Every element is tested against the
+        // tile's extent; four rows go out as one vector where all four exist unshifted and C allows it.
+        // (a k-contiguous operand has no shift: gs = the extent, sh = 0, and the tests below reduce to r < extent)
+        // The extents and the lane number pass through an empty asm: everything below is derived from them here, after
+        // the slice loop.  Otherwise the compiler computes the per-block tests up front and, with the register file full
+        // of fragments during the loop, parks them in scratch memory.
+        uint32_t e_m = m_here, e_n = n_here, e_lane = lane;
+        asm volatile("" : "+s"(e_m), "+s"(e_n), "+v"(e_lane));
+        const uint32_t gsm = TA ? e_m : (e_m - 1) / EPC * EPC, shm = TA ? 0u : gsm + EPC - e_m;
+        const uint32_t gsn = !TB ? e_n : (e_n - 1) / EPC * EPC, shn = !TB ? 0u : gsn + EPC - e_n;
+        const uint32_t vec_rows = shm == 0 ? e_m : gsm;                     // tile rows below this are in place
         const float alpha = args.alpha, beta = args.beta;
         const bool to_ws = args.splits > 1;
         float *ws = args.ws + ((size_t)split * args.batch + batch) * (size_t)args.m * args.n;
         T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
         const bool vec_c = args.vec_c != 0;
         typedef typename std::conditional<ESZ == 2, u32x2, u32x4>::type cvec;
+        const uint32_t lrow0 = wm * Cfg::TM + 4 * (e_lane >> 4), lcol0 = wn * Cfg::TN + (e_lane & 15);
         static_for<FM * FN>([&](auto IJ) {
             constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
-            const uint32_t row = wrow0 + i * 16, col = wcol0 + j * 16;
+            const uint32_t lr = lrow0 + i * 16, lc = lcol0 + j * 16;
             float v[4] = {acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
-            if (col < args.n && row < args.m) {
-                if (to_ws) {
-                    float *p = ws + (size_t)col * args.m + row;
+            // the column of C this lane's tile column stands for, if any
+            const bool col_ok = lc < gsn || (lc >= gsn + shn && lc - shn < e_n);
+            const uint32_t col = col0 + (lc < gsn ? lc : lc - shn);
+            if (col_ok) {
+                if (!to_ws && vec_c && lr + 3 < vec_rows) {
+                    T *p = C + (size_t)col * args.ldc + row0 + lr;
+                    union { T e[4]; cvec v; } io;
+                    if (beta != 0.0f) {
+                        io.v = *reinterpret_cast<const cvec *>(p);
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (row + r < args.m) p[r] = v[r];
-                } else {
-                    T *p = C + (size_t)col * args.ldc + row;
-                    if (vec_c && row + 3 < args.m) {
-                        union { T e[4]; cvec v; } io;
-                        if (beta != 0.0f) {
-                            io.v = *reinterpret_cast<const cvec *>(p);
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], alpha * v[r]);
-                        } else {
-#pragma unroll
-                            for (int r = 0; r < 4; ++r) io.e[r] = (T)(alpha * v[r]);
-                        }
-                        *reinterpret_cast<cvec *>(p) = io.v;
+                        for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], alpha * v[r]);
                     } else {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            if (row + r < args.m) {
+                        for (int r = 0; r < 4; ++r) io.e[r] = (T)(alpha * v[r]);
+                    }
+                    *reinterpret_cast<cvec *>(p) = io.v;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t tr = lr + r;
+                        const bool row_ok = tr < gsm || (tr >= gsm + shm && tr - shm < e_m);
+                        const uint32_t row = row0 + (tr < gsm ? tr : tr - shm);
+                        if (row_ok) {
+                            if (to_ws) {
+                                ws[(size_t)col * args.m + row] = v[r];
+                            } else {
+                                T *p = C + (size_t)col * args.ldc + row;
                                 float o = alpha * v[r];
-                                if (beta != 0.0f) o = __builtin_fmaf(beta, (float)p[r], o);
-                                p[r] = (T)o;
+                                if (beta != 0.0f) o = __builtin_fmaf(beta, (float)*p, o);
+                                *p = (T)o;
                             }
                         }
                     }
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);          // one block at a time: keeps the address arithmetic of 64 blocks from piling up
         });
         continue;
     }

@@ -52,13 +52,17 @@ inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_
 }
 
 // Does the ring (x16 = false) or x16 config (tile, split) take this shape?  Ring: m, n whole tiles, k whole slices, the
-// same number for every split.  x16: any shape (its loads repeat the last rows of an edge tile, its edge tiles store
-// under guards, a partial last slice of k is zero-filled; the splits take equal runs of whole slices and the last one
-// what is left, fewer splits than asked for when k is short).  Both need 16-byte aligned A and B, checked at the call.
-inline bool ring_shape_ok(int dtype, int tile, int split, size_t m, size_t n, size_t k, bool x16)
+// same number for every split; A and B 16-byte aligned (checked at the call).  x16: any shape and alignment (its loads
+// repeat or shift the last rows of an edge tile, its edge tiles store under guards, a partial last slice of k is
+// zero-filled; the splits take equal runs of whole slices and the last one what is left, fewer splits than asked for
+// when k is short) -- except a memory-contiguous m (transA = N) or n (transB = T) shorter than one 16-byte load.
+inline bool ring_shape_ok(int dtype, int tile, int split, int transA, int transB, size_t m, size_t n, size_t k, bool x16)
 {
     if (k == 0) return false;
-    if (x16) return true;
+    if (x16) {
+        const size_t per16 = dtype == MMBO_F32 ? 4 : 8;
+        return (transA || m >= per16) && (!transB || n >= per16);
+    }
     const RingRow &r = kRingTiles[tile];
     const size_t bk = (size_t)ring_bk(dtype);
     if (m % r.bm || n % r.bn || k % bk) return false;
@@ -440,8 +444,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         const bool split_lines = ((transA ? k : m) * esz) % 128 != 0 || ((transB ? n : k) * esz) % 128 != 0;
         for (int rt = 0; rt < NUM_RING_TILES; ++rt)
             for (int si = 0; si < NUM_SPLITS; ++si) {
-                const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], m, n, k, false);
-                const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], m, n, k, true);
+                const bool ring_ok = ring_shape_ok(dtype, rt, kSplits[si], transA, transB, m, n, k, false);
+                const bool x16_ok = ring_shape_ok(dtype, x16_of_ring[rt], kSplits[si], transA, transB, m, n, k, true);
                 if (!ring_ok && !x16_ok) continue;
                 // A dimension smaller than the tile: only the 64 x 64 fp16 tile on a long k is worth it (measured against
                 // the staged kernel's 32 x 32 tile: HGEMM 16 x 4096 x 4096 11.8 against 17.5 us, 48 x 48 x 8192 10.1
@@ -542,16 +546,24 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     if (config_id == MMBO_CONFIG_AUTO) {
         config_id = mmbo_select_config(dtype, transA, transB, m, n, k, batch);
         if (config_id < 0) return -config_id;
-        // The pick is made from the shape alone.  The whole-tile kernels also need 16-byte aligned A and B and a
-        // tile's span of an operand below 2 GiB: where the operands at hand do not qualify, the staged kernel
-        // (any alignment) takes the call.
+        // The pick is made from the shape alone.  The ring kernels also need 16-byte aligned A and B, every
+        // direct-to-LDS kernel a tile's span of an operand below 2 GiB: where the operands at hand do not qualify, the
+        // x16 config of the same tile and split (any alignment), or the staged kernel, takes the call.
         if (!f64) {
             const ConfigRef c = config_ref(config_id);
-            if (c.ring) {
+            if (c.ring && !c.x16) {
                 auto al16 = [&](const void *p, size_t ld, long long stride) {
                     return ((uintptr_t)p % 16 == 0) && ((ld * esz_in) % 16 == 0) && (((size_t)stride * esz_in) % 16 == 0);
                 };
-                if (!al16(A, lda, strideA) || !al16(B, ldb, strideB)) config_id = select_staged(dtype, m, n, k, batch);
+                if (!al16(A, lda, strideA) || !al16(B, ldb, strideB)) {
+                    static const int x16_of_ring[NUM_RING_TILES] = {0, 2, 3, 4};
+                    int si = 0;
+                    while (si + 1 < NUM_SPLITS && kSplits[si] != c.split) ++si;
+                    const bool wide_pick = config_id == kWideConfig;
+                    const int tile = wide_pick ? 0 : x16_of_ring[c.tile];
+                    config_id = ring_shape_ok(dtype, tile, c.split, transA, transB, m, n, k, true)
+                                    ? x16_config_id(tile, si) : select_staged(dtype, m, n, k, batch);
+                }
             }
         }
         if (!tile_span_ok(config_tile(dtype, config_id), transA, transB, lda, ldb, esz_in)) {
@@ -568,7 +580,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     int split = cref.split;
     const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
     TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0} : tile_row(dtype, cref.tile);
-    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
+    if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, transA, transB, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
     const bool wide = !f64 && config_id == kWideConfig;
     if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
@@ -607,7 +619,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     a.vec_c = aligned16(C, ldc, strideC);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (cref.ring && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
+    if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
     if (split > 1) {
         size_t bytes = (size_t)split * batch * m * n * sizeof(float);
         int rc = workspace(bytes, &a.ws);

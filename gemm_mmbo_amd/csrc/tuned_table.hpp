@@ -21,8 +21,8 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 1024, 1024, 1024, 1, 33, 93.0f},
     {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
     {0, 1, 0, 4096, 4096, 4096, 1, 51, 145.0f},
-    {0, 0, 0, 1023, 777, 513, 1, 10, 30.0f},
-    {1, 0, 0, 1023, 777, 513, 1, 10, 39.0f},
+    {0, 0, 0, 1023, 777, 513, 1, 55, 46.6f},
+    {1, 0, 0, 1023, 777, 513, 1, 55, 82.4f},
     {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
     {1, 0, 0, 4096, 128, 4096, 1, 37, 272.2f},
     {0, 0, 0, 128, 4096, 8192, 1, 45, 108.8f},

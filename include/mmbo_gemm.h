@@ -25,13 +25,13 @@
  *   - config_id selects a row of the tile-config table, like the reference's kernelId
  *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick.  Every shape runs
  *     under MMBO_CONFIG_AUTO.  Named configs: the general kernel's (no "DTL1" in the name) take any shape and
- *     alignment; the direct-to-LDS ones ("DTL1") need A and B, their leading dimensions and batch strides 16-byte
- *     aligned, and of those only the "MFMA16x16" family takes m, n that end inside a tile and k that ends inside a
- *     slice (the reference's kernels take whole tiles only: its launcher floors the grid, src/gemm/driver.h:49-50).
- *     That family fetches 16 bytes at a time: where m (transA = N) or n (transB = T) is not a whole number of such
- *     groups, the fetch of the last group of a column covers up to 14 bytes behind its last element -- padding of
- *     the leading dimension, or, for the very last column, bytes behind the matrix inside the aligned 16 bytes that
- *     hold its last element; they are read and never used;
+ *     alignment; of the direct-to-LDS ones ("DTL1") the "MFMA16x16" family takes m, n that end inside a tile, k that
+ *     ends inside a slice and A, B at any element alignment (the reference's kernels take whole tiles only: its
+ *     launcher floors the grid, src/gemm/driver.h:49-50), and reads no byte outside the operands: it fetches 16
+ *     bytes at a time, and where m (transA = N) or n (transB = T) is not a whole number of such groups the last
+ *     group of a column is the 16 bytes that end at its last element (refused, MMBO_ERR_INVALID_CONFIG, where that
+ *     dimension is shorter than one group: 4 floats, 8 halves); the others need whole tiles and A, B, their
+ *     leading dimensions and batch strides 16-byte aligned;
  *   - errors come back as status codes; nothing calls exit() (the reference's HIP_CHECK
  *     does, src/gemm/common.h:20-24).
  */

@@ -73,26 +73,23 @@ def test_cfg5_strided_batched_hgemm_tn():
 @pytest.mark.parametrize("ta", [0, 1])
 @pytest.mark.parametrize("tb", [0, 1])
 def test_every_config_every_transpose_ragged(dtype, ta, tb):
-    """257 x 131 x 1000 through every config id.  The general kernel takes it in every config.  Of the direct-to-LDS
-    kernels the ring family only takes whole tiles, and the x16 family takes this shape in TN alone (m and n odd: neither
-    may be contiguous in memory; lda = ldb = 1000 keeps the columns 16-byte aligned), with every split-K factor (31 or 62
-    whole slices and a partial one: the splits are uneven): everything else must be refused, never computed wrongly."""
+    """257 x 131 x 1000 with tightly packed operands through every config id.  The general kernel and the x16 family
+    take it in every config and transpose (odd m and n, also where they are the contiguous dimension; columns that
+    start off 16-byte boundaries; 31 or 62 whole slices of k and a partial one, split unevenly); the ring family only
+    takes whole tiles and must refuse it, never compute it wrongly."""
     import gemm_mmbo_amd as G
     taken = 0
     for cid in range(G.num_configs(dtype)):
         name = G.config_info(dtype, cid)["name"]
         p = U.Problem(dtype, ta, tb, 257, 131, 1000, 1.5, 0.5, lda=None, ldc=260, seed=10 + cid)
-        if "DTL1" in name:
-            if "MFMA16x16" in name and ta and not tb:
-                _run_and_check(p, cid, label=f"config {cid} {name}")
-                taken += 1
-                continue
+        if "DTL1" in name and "MFMA16x16" not in name:
             with pytest.raises(G.MmboError) as e:
                 U.run_gpu(p, cid)
             assert e.value.status == 5
             continue
         _run_and_check(p, cid, label=f"config {cid} {name}")
-    assert taken == (25 if ta and not tb else 0)
+        taken += "MFMA16x16" in name
+    assert taken == 25
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -207,7 +204,8 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
     a tile (loads repeat the last rows, stores are guarded: the reference's edge handling, src/gemm/ref/Kernels.cpp:
     1007-1121), down to a single row or column, odd sizes also where the dimension is the contiguous one; a k that ends
     inside a slice (zero-filled: the reference's tail loop, :921-1005), down to k smaller than one slice; with beta,
-    batches, and padded leading dimensions whose padding rows of C must stay untouched."""
+    batches, padded leading dimensions whose padding rows of C must stay untouched, and operands whose columns start off
+    16-byte boundaries (the direct loads take any element-aligned address)."""
     import gemm_mmbo_amd as G
     bk = 16 if dtype == F32 else 32
     g = 4 if dtype == F32 else 8                                # elements per 16 bytes
@@ -224,20 +222,31 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
         # m, n that end inside a 16-byte group (also where that dimension is the contiguous one) and inside a 4-row group
         cases += [(bm + 3, bn + g, 5, -1.0, 1.0, 1, 0, 0), (bm + g, bn - 1, 6, 1.0, 0.5, 1, 0, 3), (bm - 1, 2 * bn + 1, 4, 1.0, 0.0, 2, 8, 7),
                   (1, 1, 1, 1.0, 0.0, 1, 0, 1), (bm + g + 1, 3, 2, 1.5, 0.5, 1, 8, 0)]
-        for (m, n, slices, alpha, beta, batch, pad, kt) in cases:
+        cases = [c + (True,) for c in cases]
+        # tightly packed or oddly padded operands at element offsets: columns of A and B start off 16-byte boundaries
+        cases += [(bm + 3, bn + 5, 3, 1.0, 0.0, 1, 0, 1, False), (2 * bm - 1, bn - 7, 2, 1.5, 0.5, 2, 0, bk - 3, False),
+                  (g + 1, bn + 1, 1, 1.0, 1.0, 1, 0, 0, False), (bm + 1, g, 5, 1.0, 0.0, 1, 0, 5, False), (bm, bn, 4, 1.0, 0.0, 1, 0, 0, False)]
+        for (m, n, slices, alpha, beta, batch, pad, kt, aligned) in cases:
             k = bk * slices * sp + kt
             ar, br = U.stored_shape(ta, m, k)[0], U.stored_shape(tb, k, n)[0]
-            lda, ldb = -(-ar // g) * g + pad, -(-br // g) * g + pad       # columns of A and B start on 16-byte boundaries
+            if aligned:
+                lda, ldb = -(-ar // g) * g + pad, -(-br // g) * g + pad   # columns of A and B start on 16-byte boundaries
+            else:
+                lda, ldb = ar + cid % 2, br + (cid % 3 == 0)
+            if (not ta and m < g) or (tb and n < g):
+                continue                                                # a contiguous dimension shorter than one load: refused
             p = U.Problem(dtype, ta, tb, m, n, k, alpha, beta, lda=lda, ldb=ldb, ldc=m + (3 if pad else 0), batch=batch,
                           seed=900 + cid + slices, dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
-            _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch}")
+            _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch} ld {lda},{ldb}",
+                           offsets=(0, 0, 0) if aligned else (1, 3, 1))
             ran += 1
-    assert ran >= 25 * 13
+    assert ran >= 25 * 16
 
 
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
-    ragged border of tiles, against the oracle.  Unaligned operands are refused; ld > dim and the automatic pick work."""
+    ragged border of tiles, against the oracle.  Unaligned operands are taken, a contiguous dimension shorter than one
+    16-byte load is refused; ld > dim and the automatic pick work."""
     import gemm_mmbo_amd as G
     ids = _x16_ids()
     for cid in ids[:2]:
@@ -246,13 +255,18 @@ def test_x16_kernel_chip_block_order_and_refusals():
             p = U.Problem(F16, 0, 0, m, n, k, 1.0, 0.0, seed=300 + m // 256, dist="normal", c_fill="nan")
             _run_and_check(p, cid, label=f"chip blocks {m}x{n}x{k}")
     cid = ids[0]
-    # unaligned A or B (an element offset, a leading dimension that is not a whole number of 16-byte groups)
+    # unaligned A or B (an element offset, a leading dimension that is not a whole number of 16-byte groups) are taken
     for (dtype, ta, tb, m, n, k, offs) in ((F16, 0, 0, 256, 256, 128, (1, 0, 0)), (F16, 0, 0, 256, 256, 128, (0, 4, 0)),
-                                           (F16, 0, 0, 255, 256, 128, (0, 0, 0)), (F32, 0, 1, 256, 254, 136, (0, 0, 0))):
+                                           (F16, 0, 0, 255, 256, 128, (0, 0, 0)), (F32, 0, 1, 256, 254, 136, (3, 1, 0))):
+        p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.0, seed=5, c_fill="nan", dist="normal" if dtype == F16 else "uniform")
+        _run_and_check(p, _x16_ids(dtype)[0], label=f"x16 unaligned {m}x{n}x{k} {offs}", offsets=offs)
+    # refused: a memory-contiguous m or n shorter than one 16-byte load
+    for (dtype, ta, tb, m, n, k) in ((F16, 0, 0, 7, 256, 128), (F16, 1, 1, 256, 5, 128), (F32, 0, 1, 3, 3, 64)):
         p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.0, seed=5, c_fill="nan")
         with pytest.raises(G.MmboError) as e:
-            U.run_gpu(p, cid, offs)
+            U.run_gpu(p, _x16_ids(dtype)[0])
         assert e.value.status == 5
+        _run_and_check(p, -1, label="auto on a thin contiguous dimension")
     p = U.Problem(F16, 1, 0, 512, 512, 320, 1.0, 0.5, lda=1032, ldb=1040, ldc=520, seed=71, dist="normal")
     _run_and_check(p, cid, label="x16 ld>dim")
     # C needs no alignment: an odd element offset and an odd ldc take the element-wise epilogue, with and without beta
@@ -271,7 +285,7 @@ def test_x16_kernel_chip_block_order_and_refusals():
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_ring_kernel_refuses_shapes_it_cannot_take(dtype):
     """Ragged m/n, k that does not split into whole slices, unaligned A: MMBO_ERR_INVALID_CONFIG, never a wrong
-    result; the automatic pick falls back to the staged kernel and still matches the oracle."""
+    result; the automatic pick moves to a kernel that takes the problem and still matches the oracle."""
     import gemm_mmbo_amd as G
     cid = _ring_ids(dtype)[0]
     bk = 16 if dtype == F32 else 32
@@ -495,23 +509,30 @@ def test_offline_tuner_emits_table_rows_for_small_shapes():
 
 
 def test_automatic_pick_never_fails_on_its_own_choice():
-    """MMBO_CONFIG_AUTO picks from the shape; the whole-tile kernels also need 16-byte aligned A and B and a tile span
-    below 2 GiB.  With operands that do not qualify the call must still succeed (staged kernel), while naming the
-    whole-tile config explicitly is refused."""
+    """MMBO_CONFIG_AUTO picks from the shape; the ring kernels also need 16-byte aligned A and B, every direct-to-LDS
+    kernel a tile span below 2 GiB.  With operands that do not qualify the call must still succeed (the x16 twin of the
+    pick, or the general kernel), while naming the config explicitly is refused."""
     import torch
 
     import gemm_mmbo_amd as G
-    # a whole-tile shape whose pick is a direct-to-LDS config, A (then B) one element off 16-byte alignment
-    for dtype in (F16, F32):
-        m, n, k = 1024, 1024, 512
-        cid = G.select_config(dtype, 0, 0, m, n, k)
-        assert "DTL1" in G.config_info(dtype, cid)["name"]
-        for offs in ((1, 0, 0), (0, 1, 0)):
-            p = U.Problem(dtype, 0, 0, m, n, k, 1.0, 0.0, seed=90, dist="normal" if dtype == F16 else "uniform", c_fill="nan")
-            with pytest.raises(G.MmboError) as e:
-                U.run_gpu(p, cid, offs)
-            assert e.value.status == 5
-            _run_and_check(p, -1, label=f"auto with unaligned operand {offs}", offsets=offs)
+    # a whole-tile fp32 shape whose pick is a ring config, A (then B) one element off 16-byte alignment
+    m, n, k = 1024, 1024, 512
+    cid = G.select_config(F32, 0, 0, m, n, k)
+    name = G.config_info(F32, cid)["name"]
+    assert "DTL1" in name and "MFMA16x16" not in name
+    for offs in ((1, 0, 0), (0, 1, 0)):
+        p = U.Problem(F32, 0, 0, m, n, k, 1.0, 0.0, seed=90, c_fill="nan")
+        with pytest.raises(G.MmboError) as e:
+            U.run_gpu(p, cid, offs)
+        assert e.value.status == 5
+        _run_and_check(p, -1, label=f"auto with unaligned operand {offs}", offsets=offs)
+    # an fp16 pick that is an x16 config takes unaligned operands by name
+    m, n, k = 2048, 2048, 1024
+    cid = G.select_config(F16, 0, 0, m, n, k)
+    assert "MFMA16x16" in G.config_info(F16, cid)["name"]
+    for offs in ((1, 0, 0), (0, 1, 0)):
+        p = U.Problem(F16, 0, 0, m, n, k, 1.0, 0.0, seed=90, dist="normal", c_fill="nan")
+        _run_and_check(p, cid, label=f"x16 by name with unaligned operand {offs}", offsets=offs)
     # a leading dimension so large that the rows of A^T under the picked tile span more than 2 GiB (only the first k rows of
     # each stored column are used): the pick itself is refused by name, the automatic path moves to a tile that fits
     m, n, k = 64, 16384, 100
@@ -539,8 +560,8 @@ def test_automatic_pick_never_fails_on_its_own_choice():
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_large_ragged_problems_through_the_automatic_pick(dtype):
     """MMBO_CONFIG_AUTO on large shapes that are not made of whole tiles: one launch of the x16 kernel (edge tiles, a
-    zero-filled last slice of k, contiguous dimensions that end inside a 16-byte group), the general kernel where A or
-    B is not 16-byte aligned.  Against the oracle, with beta, ld > dim (padding rows untouched), every transpose, batches,
+    zero-filled last slice of k, contiguous dimensions that end inside a 16-byte group, columns that start off 16-byte
+    boundaries).  Against the oracle, with beta, ld > dim (padding rows untouched), every transpose, batches,
     bit-identical on repetition."""
     import gemm_mmbo_amd as G
     dist = "normal" if dtype == F16 else "uniform"
@@ -556,7 +577,7 @@ def test_large_ragged_problems_through_the_automatic_pick(dtype):
         got = _run_and_check(p, -1, label=f"ragged {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} {kw}")
         again, _ = U.run_gpu(p, -1)
         assert np.array_equal(got.view(U.BITS[dtype]), again.view(U.BITS[dtype]))
-    # unaligned A: one launch of the general kernel, same result bar
+    # unaligned A
     p = U.Problem(dtype, 0, 0, 2100, 2300, 2560, 1.0, 0.0, seed=77, dist=dist, c_fill="nan")
     _run_and_check(p, -1, label="ragged, unaligned A", offsets=(1, 0, 0))
 
@@ -564,7 +585,8 @@ def test_large_ragged_problems_through_the_automatic_pick(dtype):
 def test_random_shapes_paddings_and_configs_against_the_oracle():
     """240 seeded random problems: both element types, every transpose, m, n, k from 1 up (a few thousand for some),
     leading dimensions padded, tight or off 16-byte alignment, batches, alpha/beta variants, through MMBO_CONFIG_AUTO
-    or a random x16 config id.  A named config may refuse the problem (status 5); whatever runs must match the oracle
+    or a random x16 config id.  A named config may refuse the problem (status 5: a contiguous dimension shorter than
+    one 16-byte load); whatever runs must match the oracle
     and leave the padding rows and the guard words behind C untouched."""
     import random
 
@@ -600,4 +622,4 @@ def test_random_shapes_paddings_and_configs_against_the_oracle():
         U.check(p, got, label)
         assert np.all(guard == 0), label
         ran += 1
-    assert ran >= 150 and refused >= 10
+    assert ran >= 200
