@@ -11,8 +11,8 @@ GPU it runs on:
     python -m gemm_mmbo_amd.tune shapes.txt --dump t.json    # also write every config's time per shape
 
 For every shape it prints the ranking and one line in the table's syntax; paste the lines into kTuned[] and rebuild.
-Configs that do not apply to a shape (the ring kernels on ragged shapes, every direct-to-LDS kernel on operands that are
-not 16-byte aligned: the operands here are tightly packed) are skipped, as the C ABI refuses them.
+Configs that do not apply to a shape (the ring kernels on ragged shapes or on operands that are not 16-byte aligned: the
+operands here are tightly packed) are skipped, as the C ABI refuses them.
 """
 import sys
 
