@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmmbo_gemm.so")
 
 EXPORTS = (
     "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
-    "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
+    "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_batch_xcd_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
 
@@ -67,6 +67,8 @@ def lib():
         L.mmbo_wg_remap.restype = ci
         L.mmbo_chip_block_remap.argtypes = [cu, cu, cu, ctypes.POINTER(cu), ctypes.POINTER(cu)]
         L.mmbo_chip_block_remap.restype = ci
+        L.mmbo_batch_xcd_remap.argtypes = [cu, cu, cu, ctypes.POINTER(cu), ctypes.POINTER(cu)]
+        L.mmbo_batch_xcd_remap.restype = ci
         L.mmbo_release_workspace.restype = ci
         dp = ctypes.POINTER(ctypes.c_double)
         L.mmbo_probe_mfma_ceiling.argtypes = [ci, ci, dp, dp]
@@ -148,6 +150,13 @@ def select_config(dtype, transA, transB, m, n, k, batch=1):
 def wg_remap(linear_id, nwg0, nwg1, wgm=8, num_xcd=8):
     a, b = ctypes.c_uint(0), ctypes.c_uint(0)
     _check(lib().mmbo_wg_remap(linear_id, nwg0, nwg1, wgm, num_xcd, ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value
+
+
+def batch_xcd_remap(linear_id, tiles, batch):
+    """(tile, batch index) of a work-group of a batch of small problems laid out one problem per XCD."""
+    a, b = ctypes.c_uint(0), ctypes.c_uint(0)
+    _check(lib().mmbo_batch_xcd_remap(linear_id, tiles, batch, ctypes.byref(a), ctypes.byref(b)))
     return a.value, b.value
 
 

@@ -44,6 +44,7 @@ struct GemmArgs {
     uint32_t batch;
     uint32_t vec_a, vec_b, vec_c;   // 1 when 128-bit accesses to that operand are aligned
     uint32_t chip_block;    // 1: tiles are walked in 16 x 16 chip-wide blocks (chip_block_remap) instead of wg_remap
+    uint32_t batch_xcd;     // 1: every problem of the batch runs on one XCD (batch_xcd_remap)
 };
 
 // Linear work-group id -> (tile row, tile column).
@@ -72,6 +73,30 @@ __host__ __device__ inline void wg_remap(uint32_t id, uint32_t nwg0, uint32_t nw
     uint32_t width = rem == 0 ? wgm : rem;
     wg0 = serial / width;
     wg1 = serial % width + block * wgm;
+}
+
+// Batches of small problems: linear dispatch index (x + tiles * z, the order the hardware hands work-groups to the
+// XCDs round-robin) -> (tile, batch index) such that all tiles of one problem run on one XCD, one after the other in
+// that XCD's share of the dispatch order.  The dispatcher's own order spreads a problem with fewer tiles than XCDs over
+// as many XCDs as it has tiles: no two work-groups that read the same panel of A or B share an L2, and every panel
+// comes from memory once per work-group that reads it (HGEMM TN 64 x 512^3 on 256 x 256 tiles: 128 MB of operand
+// reads instead of 64).  Requires batch % nxcd == 0; a bijection of [0, tiles * batch).
+__host__ __device__ inline void batch_xcd_remap(uint32_t lin, uint32_t tiles, uint32_t nxcd, uint32_t &tile, uint32_t &z)
+{
+    const uint32_t x = lin % nxcd, slot = lin / nxcd;
+    z = (slot / tiles) * nxcd + x;
+    tile = slot % tiles;
+}
+
+// What a work-group does: (tile id for wg_remap, z = split * batch + batch index, XCD count for wg_remap) from its
+// block indices.  bx = blockIdx.x (or the tile a resident work-group has walked to), bz = blockIdx.z.
+__device__ inline void work_of_block(const GemmArgs &args, uint32_t bx, uint32_t bz, uint32_t &tile, uint32_t &z, uint32_t &nxcd)
+{
+    tile = bx; z = bz; nxcd = args.nxcd;
+    if (args.batch_xcd) {
+        batch_xcd_remap(bx + args.nwg0 * args.nwg1 * bz, args.nwg0 * args.nwg1, args.nxcd, tile, z);
+        nxcd = 1;                                       // the tiles of one problem are on one XCD already
+    }
 }
 
 // Linear work-group id -> (tile row, tile column) in chip-wide blocks, for a chip of 8 XCDs x 32 CUs that runs one

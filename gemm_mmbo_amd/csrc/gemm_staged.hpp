@@ -196,9 +196,9 @@ gemm_staged_kernel(const GemmArgs args)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
 
-    uint32_t wg0, wg1;
-    wg_remap(blockIdx.x, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
-    const uint32_t zb = blockIdx.z;
+    uint32_t wg0, wg1, tile_id, zb, nxcd;
+    work_of_block(args, blockIdx.x, blockIdx.z, tile_id, zb, nxcd);
+    wg_remap(tile_id, args.nwg0, args.nwg1, args.wgm, nxcd, wg0, wg1);
     const uint32_t split = zb / args.batch, batch = zb % args.batch;
 
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;

@@ -319,10 +319,14 @@ gemm_x16_kernel(const GemmArgs args)
     // only ever wait for more when something older is still outstanding.
     const uint32_t n_tiles = args.nwg0 * args.nwg1;
     for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    uint32_t wg0, wg1;
-    if (args.chip_block) chip_block_remap(tile, args.nwg0, args.nwg1, wg0, wg1);
-    else wg_remap(tile, args.nwg0, args.nwg1, args.wgm, args.nxcd, wg0, wg1);
-    const uint32_t zb = blockIdx.z;
+    uint32_t wg0, wg1, tile_id, zb, nxcd;
+    work_of_block(args, tile, blockIdx.z, tile_id, zb, nxcd);
+    if (args.chip_block) chip_block_remap(tile_id, args.nwg0, args.nwg1, wg0, wg1);
+    else wg_remap(tile_id, args.nwg0, args.nwg1, args.wgm, nxcd, wg0, wg1);
+    // (the divisions above run on the vector unit; what follows wants these in scalar registers)
+    wg0 = __builtin_amdgcn_readfirstlane(wg0);
+    wg1 = __builtin_amdgcn_readfirstlane(wg1);
+    zb = __builtin_amdgcn_readfirstlane(zb);
     const uint32_t split = zb / args.batch, batch = zb % args.batch;
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
     const uint32_t lda = args.lda, ldb = args.ldb;

@@ -494,6 +494,18 @@ int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsi
     return MMBO_OK;
 }
 
+int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, unsigned *tile, unsigned *batch_index)
+{
+    if (!tile || !batch_index) return MMBO_ERR_NULL_POINTER;
+    if (tiles == 0 || batch == 0 || batch % 8 != 0) return MMBO_ERR_INVALID_SIZE;
+    if ((unsigned long long)tiles * batch > 0xFFFFFFFFull || linear_id >= tiles * batch) return MMBO_ERR_INVALID_SIZE;
+    uint32_t t, z;
+    batch_xcd_remap(linear_id, tiles, 8, t, z);
+    *tile = t;
+    *batch_index = z;
+    return MMBO_OK;
+}
+
 int mmbo_release_workspace(void)
 {
     int dev = 0;
@@ -611,6 +623,8 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     a.k_per_split = (uint32_t)(split > 1 ? k_per_split : (k ? k : 1));
     a.batch = (uint32_t)batch;
     a.chip_block = cref.x16 && r.bm == 256 && r.bn == 256 && nwg0 >= 16 && nwg1 >= 16;
+    // batches of problems of at most 32 tiles (an XCD's CUs hold them at one time): each problem on one XCD
+    a.batch_xcd = split == 1 && batch >= a.nxcd && batch % a.nxcd == 0 && nwg0 * nwg1 <= 32;
     auto aligned16 = [&](const void *p, size_t ld, long long stride) {
         return ((uintptr_t)p % 16 == 0) && ((ld * esz) % 16 == 0) && (((size_t)stride * esz) % 16 == 0);
     };

@@ -123,6 +123,13 @@ int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm
  * A bijection of [0, nwg0*nwg1); needs nwg0 >= 16 and nwg1 >= 16.  Pure host logic. */
 int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned *wg0, unsigned *wg1);
 
+/* Host twin of how a batch of small problems (at most 32 tiles each, batch a multiple of 8, no split-K) is laid over
+ * the chip: linear dispatch index (tile slot + tiles * z, the order in which the hardware hands work-groups to its 8
+ * XCDs round-robin) -> (tile, batch index), all tiles of one problem on one XCD so that the work-groups that read the
+ * same panel of A or B share an L2.  The reference has no batches in its launcher (src/gemm/driver.h:49-59) and one
+ * L2.  A bijection of [0, tiles*batch); needs batch % 8 == 0.  Pure host logic. */
+int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, unsigned *tile, unsigned *batch_index);
+
 /* Release the split-K workspace held for the current device (allocated lazily, grown on
  * demand, reused across calls).  The reference never frees what it loads (src/gemm/driver.h:41). */
 int mmbo_release_workspace(void);

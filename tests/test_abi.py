@@ -140,6 +140,24 @@ def test_chip_block_remap_bijection_and_block_structure(nwg0, nwg1):
         prev = (r0, c0)
 
 
+@pytest.mark.parametrize("tiles,batch", [(4, 64), (1, 8), (16, 16), (32, 24), (3, 40)])
+def test_batch_xcd_remap_bijection_and_one_problem_per_xcd(tiles, batch):
+    """Batches of small problems: a bijection of the dispatch indices onto (tile, batch index); all tiles of one
+    problem fall on one XCD (dispatch index % 8), on consecutive turns of that XCD."""
+    got = [G.batch_xcd_remap(lid, tiles, batch) for lid in range(tiles * batch)]
+    assert sorted(got) == [(t, z) for t in range(tiles) for z in range(batch)]
+    for z in range(batch):
+        lids = [lid for lid, (t, zz) in enumerate(got) if zz == z]
+        assert len({lid % 8 for lid in lids}) == 1
+        turns = sorted(lid // 8 for lid in lids)
+        assert turns == list(range(turns[0], turns[0] + tiles))
+        assert [got[lid][0] for lid in sorted(lids)] == list(range(tiles))
+    with pytest.raises(G.MmboError):
+        G.batch_xcd_remap(0, tiles, batch + 1)
+    with pytest.raises(G.MmboError):
+        G.batch_xcd_remap(tiles * batch, tiles, batch)
+
+
 def test_chip_block_remap_rejects_bad_arguments():
     with pytest.raises(G.MmboError):
         G.chip_block_remap(0, 15, 16)        # fewer than 16 tile rows

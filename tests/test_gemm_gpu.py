@@ -67,6 +67,44 @@ def test_cfg5_strided_batched_hgemm_tn():
     _run_and_check(p, label="cfg5")
 
 
+def test_batches_of_small_problems_one_per_xcd():
+    """Batches that are multiples of 8, of problems of at most 32 tiles: every kernel family lays one problem on one
+    XCD (mmbo_batch_xcd_remap) instead of the dispatcher's order.  Every GlobalSplitU = 1 config of each family (fp32,
+    fp16) and the fp64 configs, 1 to 32 tiles per problem, ragged sizes for the kernels that take them, gaps between
+    the matrices of the batch, beta != 0; and neighbours that must stay on the plain order (batch 12, 36 tiles, split-K)."""
+    import gemm_mmbo_amd as G
+    ran = 0
+    for dtype in (F32, F16, U.F64):
+        dist = "normal" if dtype == F16 else "uniform"
+        for cid in range(G.num_configs(dtype)):
+            d = G.config_info(dtype, cid)
+            name = d["name"]
+            ring_only = "DTL1" in name and "_ACC" not in name
+            if "GSU01" not in name or ("+3U" in name and dtype != F16):
+                continue
+            bm, bn = d["macro_tile_m"], d["macro_tile_n"]
+            bk = 64 if "+3U" in name else d["depth_u"]
+            shapes = [(bm, bn, 4 * bk, 8), (2 * bm, 2 * bn, 2 * bk, 16), (4 * bm, 8 * bn, 2 * bk, 8)]
+            if not ring_only and bm <= 128:
+                shapes.append((2 * bm - 3, 3 * bn - 5, 3 * bk + 1, 24))
+            for (m, n, k, batch) in shapes:
+                if m * n * batch > 48 << 20:
+                    continue
+                ta, tb = (cid % 2, (cid // 2) % 2) if "+3U" not in name else (0, 0)
+                k = max(k, 512) if "+3U" in name else k             # the wide-unit kernel needs k >= 512
+                (ar, ac), (br, bc) = U.stored_shape(ta, m, k), U.stored_shape(tb, k, n)
+                gap = 0 if "+3U" in name else 8
+                p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.5, batch=batch, seed=40 + cid, dist=dist, c_fill="uniform",
+                              strides=(ar * ac + gap, br * bc + gap, m * n + gap))
+                _run_and_check(p, cid, label=f"{name} {m}x{n}x{k} b{batch}")
+                ran += 1
+    assert ran >= 60
+    for (dtype, m, n, k, batch, cid) in ((F16, 256, 256, 256, 12, -1), (F16, 384, 384, 128, 8, _x16_ids(F16)[4]),
+                                         (F32, 128, 128, 512, 8, _x16_ids(F32)[4 + 5])):
+        p = U.Problem(dtype, 1, 0, m, n, k, 1.0, 1.0, batch=batch, seed=3, dist="normal" if dtype == F16 else "uniform", c_fill="uniform")
+        _run_and_check(p, cid, label=f"plain order {m}x{n}x{k} b{batch}")
+
+
 # ------------------------------------------------------------------ every config id on ragged shapes
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
