@@ -199,6 +199,50 @@ def ragged_legs(G, torch, steps, warmup):
     return out
 
 
+def config_legs(G, torch, steps, warmup):
+    """The benchmark configurations that are not the headline: SGEMM NN 1024^3 (alpha = 1, beta = 0), SGEMM NT and TN
+    4096^3 (alpha = 1.5, beta = 0.5) and the strided-batched HGEMM TN 64 x 512^3 (alpha = 1, beta = 1), one launch each
+    through the automatic pick, timed with events on the launch stream.  Algorithmic bytes count C twice where
+    beta != 0.  Parity of these configurations is in tests/test_gemm_gpu.py."""
+    stream = torch.cuda.current_stream()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    out = {}
+    for key, dtype, tdt, ta, tb, m, n, k, batch, alpha, beta in (
+            ("cfg1_sgemm_nn_1024", G.F32, torch.float32, 0, 0, 1024, 1024, 1024, 1, 1.0, 0.0),
+            ("cfg2a_sgemm_nt_4096", G.F32, torch.float32, 0, 1, 4096, 4096, 4096, 1, 1.5, 0.5),
+            ("cfg2b_sgemm_tn_4096", G.F32, torch.float32, 1, 0, 4096, 4096, 4096, 1, 1.5, 0.5),
+            ("cfg5_hgemm_tn_512_batch64", G.F16, torch.float16, 1, 0, 512, 512, 512, 64, 1.0, 1.0)):
+        scale = 0.1 if dtype == G.F16 else 1.0
+        A = ((torch.rand(m * k * batch, device="cuda", generator=gen) * 2 - 1) * scale).to(tdt)
+        B = ((torch.rand(k * n * batch, device="cuda", generator=gen) * 2 - 1) * scale).to(tdt)
+        C = (torch.rand(m * n * batch, device="cuda", generator=gen) * 2 - 1).to(tdt)
+        lda, ldb = (k if ta else m), (n if tb else k)
+        cid = G.select_config(dtype, ta, tb, m, n, k, batch)
+
+        def run():
+            G.gemm_strided_batched(dtype, ta, tb, m, n, k, alpha, A, lda, m * k, B, ldb, k * n, beta, C, m, m * n, batch,
+                                   G.CONFIG_AUTO, stream)
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            run()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / steps * 1e3
+        tf = 2.0 * m * n * k * batch / us * 1e-6
+        esz = 2 if dtype == G.F16 else 4
+        gbps = batch * (m * k + k * n + m * n * (2 if beta != 0 else 1)) * esz / us * 1e-3
+        out[key] = {"us": round(us, 1), "tflops": round(tf, 1),
+                    "frac_of_peak": round(tf / PEAK_TFLOPS["f16" if dtype == G.F16 else "f32"], 4),
+                    "algorithmic_GBps": round(gbps, 1), "tile_config": G.config_info(dtype, cid)["name"]}
+        del A, B, C
+    return out
+
+
 def cpu_baseline(dtype, m, n, k, hA, hB):
     """The oracle's native-precision CPU GEMM (fp16 operands widened to fp32, fp32 multiply-add chains) on
     the same operands, all host cores, whole problem once."""
@@ -277,6 +321,7 @@ def main():
     f64 = dgemm_legs(G, torch, args.steps, args.warmup) if args.only in (None, "f64") else {}
     skinny = skinny_legs(G, torch, args.steps, args.warmup) if not args.only else {}
     ragged = ragged_legs(G, torch, min(args.steps, 10), min(args.warmup, 3)) if not args.only else {}
+    configs = config_legs(G, torch, min(args.steps, 20), min(args.warmup, 5)) if not args.only else {}
     if args.only == "f64":
         print(json.dumps({"metric": METRIC, "also": f64}))
         return
@@ -326,6 +371,8 @@ def main():
         out.setdefault("also", {})["skinny_nn_hbm_bound"] = skinny
     if ragged:
         out.setdefault("also", {})["ragged_one_launch"] = ragged
+    if configs:
+        out.setdefault("also", {})["other_benchmark_configs"] = configs
     if f64:
         out.setdefault("also", {}).update(f64)
         out["parity_ok"] = bool(out["parity_ok"] and f64["fp64_hpl_max_rel_err"] <= f64["fp64_hpl_rel_err_limit"]
