@@ -22,7 +22,7 @@ PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}      # MI355X published
 # Bytes per launch that crossed the L2 <-> fabric boundary, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
 # this same command (each scaled by the counter's reading for a plain elementwise pass of known size; the
 # summaries with the commands are profiles/gemm_x16_f16_8192.txt and profiles/gemm_x16_f32_8192.txt).
-MEASURED_TRAFFIC_BYTES = {"f16": 1.635e9 + 0.135e9, "f32": 3.236e9 + 0.319e9}
+MEASURED_TRAFFIC_BYTES = {"f16": 1.626e9 + 0.135e9, "f32": 3.231e9 + 0.335e9}
 
 
 def time_gemm(G, torch, dtype, m, n, k, steps, warmup, seed):
