@@ -303,7 +303,8 @@ gemm_ring_kernel(const GemmArgs args)
     // slice has the larger the exposed share: measured on fp32 4096 x 128 x 4096, reads spread over the whole slice
     // cost 10 us on top of 35 us of MFMAs.
     constexpr int READ_SPAN = Cfg::NW > 4 ? NMFMA : (NMFMA >= 32 ? NMFMA * 3 / 4 : NMFMA / 2);
-    auto mfma_and_read = [&](const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
+    auto mfma_and_read = [&](auto ALWAYS, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
+        constexpr bool always = decltype(ALWAYS)::value;          // steady state: every slice issues its loads, no flag test
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         char *dst = lds + lbuf * Cfg::SLICE_BYTES;
         const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
@@ -337,7 +338,7 @@ gemm_ring_kernel(const GemmArgs args)
                 static_for<l1 - l0>([&](auto LL) {
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < BATCH) {
-                        if (load) {
+                        if (always || load) {
                             if constexpr (l < TileA::LPW)
                                 __builtin_amdgcn_global_load_lds(
                                     (const __attribute__((address_space(1))) void *)(pa + offA[l]),
@@ -383,18 +384,33 @@ gemm_ring_kernel(const GemmArgs args)
     MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
 
     int buf = 0;                                                     // s % DEPTH
+    // steady state: every slice issues its loads; no flag is tested inside the loop (with two MFMAs per slice in the
+    // smallest fp16 tile the tests and branches were a third of the instructions a wavefront issued per slice)
+    auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
+        const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
+        mfma_and_read(std::true_type{}, ca, cb, na, nb, nbuf, true, s + DEPTH, buf);
+        MMBO_WAIT_LGKM0();
+        MMBO_WAIT_VM(BATCH * (DEPTH - 2));
+        MMBO_BARRIER();
+        buf = nbuf;
+    };
     auto step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
         const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
         const bool steady = s + DEPTH < n_slice;
         // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
         // interleaved block free of divergent control flow)
-        mfma_and_read(ca, cb, na, nb, nbuf, steady, s + DEPTH, buf);
+        mfma_and_read(std::false_type{}, ca, cb, na, nb, nbuf, steady, s + DEPTH, buf);
         MMBO_WAIT_LGKM0();
         if (steady) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();
         buf = nbuf;
     };
-    for (int s = 0; s < n_slice; s += 2) {
+    int s = 0;
+    for (; s + 1 + DEPTH < n_slice; s += 2) {
+        steady_step(s, fa[0], fb[0], fa[1], fb[1]);
+        steady_step(s + 1, fa[1], fb[1], fa[0], fb[0]);
+    }
+    for (; s < n_slice; s += 2) {
         step(s, fa[0], fb[0], fa[1], fb[1]);
         if (s + 1 < n_slice) step(s + 1, fa[1], fb[1], fa[0], fb[0]);
     }

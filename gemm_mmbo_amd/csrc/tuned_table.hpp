@@ -26,7 +26,7 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
     {1, 0, 0, 4096, 128, 4096, 1, 37, 272.2f},
     {0, 0, 0, 128, 4096, 8192, 1, 45, 108.8f},
-    {1, 0, 0, 128, 4096, 8192, 1, 64, 398.7f},
+    {1, 0, 0, 128, 4096, 8192, 1, 40, 423.9f},
     {1, 1, 0, 512, 512, 512, 64, 51, 442.8f},
     {0, 0, 0, 2048, 2048, 2048, 1, 33, 117.5f},
     {1, 0, 0, 2048, 2048, 2048, 1, 53, 761.2f},
