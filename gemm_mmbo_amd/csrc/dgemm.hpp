@@ -212,11 +212,7 @@ dgemm_kernel(const GemmArgs args)
     __syncthreads();
 
     int cur = 0;
-    for (int it = 0; it < n_iter; ++it) {
-        const bool more = it + 1 < n_iter;
-        if (more) load_stage(it + 1);
-
-        const char *st = lds + cur * Cfg::STAGE_BYTES;
+    auto multiply_stage = [&](const char *st) {
 #pragma unroll
         for (int kk = 0; kk < NKK; ++kk) {
             double fa[FM], fb[FN];
@@ -230,6 +226,27 @@ dgemm_kernel(const GemmArgs args)
                 for (int j = 0; j < FN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
+    };
+    int it = 0;
+    if (fast) {
+        // interior tiles of aligned operands, while the next stage is a whole one: no test inside the loop, the
+        // predicated loader stays out of its body
+        for (; it + 1 < n_full; ++it) {
+            TileA::load_fast(ra, gA + (int64_t)(it + 1) * stepA, offA);
+            TileB::load_fast(rb, gB + (int64_t)(it + 1) * stepB, offB);
+            multiply_stage(lds + cur * Cfg::STAGE_BYTES);
+            char *nx = lds + (cur ^ 1) * Cfg::STAGE_BYTES;
+            TileA::store_lds(ra, nx, tid);
+            TileB::store_lds(rb, nx + TileA::LDS_BYTES, tid);
+            __syncthreads();
+            cur ^= 1;
+        }
+    }
+    for (; it < n_iter; ++it) {
+        const bool more = it + 1 < n_iter;
+        if (more) load_stage(it + 1);
+
+        multiply_stage(lds + cur * Cfg::STAGE_BYTES);
 
         if (more) {
             char *nx = lds + (cur ^ 1) * Cfg::STAGE_BYTES;
