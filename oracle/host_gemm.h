@@ -26,7 +26,12 @@
  *     exact power-of-two inputs, transpose identity (A*B)^T = B^T*A^T, numpy float64
  *     matmul as a second opinion, committed fixtures under tests/golden/;
  *   - fp16 conversion: numpy.float16 over every 16-bit pattern and random floats;
- *   - RNG: an independent numpy restatement of the same counter construction.
+ *   - RNG: an independent numpy restatement of the same counter construction;
+ *   - the comparator oracle_max_rel_err (counterpart of the reference's compare loop, src/gemm/test.cc:109-120):
+ *     fed results that are wrong in known ways -- one element off by a known amount anywhere in the buffer, NaN and
+ *     Inf, garbage in padding rows and batch gaps, a wrong leading dimension or batch stride -- it must report exactly
+ *     the expected error; a comparator that dropped its NaN rule, a stride, a batch, its floor or its max-reduction
+ *     fails those tests.
  *   No function here is "parity unpinned".
  */
 #ifndef ORACLE_HOST_GEMM_H

@@ -277,3 +277,143 @@ def test_bad_arguments_rejected():
         O.gemm_f64(F32, 0, 0, 4, 4, 4, 1.0, A, 3, A, 4, 0.0, None, 4)      # lda < m
     with pytest.raises(ValueError):
         O.gemm_f64(F32, 0, 0, 4, 4, 4, 1.0, A, 4, A, 4, 0.0, None, 3)      # ldc < m
+
+
+# ------------------------------------------------------------------ the comparator itself
+# Every tolerance assertion of the parity tests goes through oracle_max_rel_err (the counterpart of the reference's
+# compare loop, src/gemm/test.cc:109-120).  These tests feed it results that are wrong in known ways and check that it
+# says so: a comparator that overlooked NaNs, a stride, a batch or its own floor would make every parity test pass
+# vacuously.
+
+def _cmp_case(dtype, m=7, n=5, ldg=11, batch=3, gap=13, seed=21):
+    """want (dense fp64, exactly representable in dtype) and a got buffer (ldg > m, batch stride > ldg*n) that
+    holds the same values, padding and gaps filled with a sentinel."""
+    npdt = O.np_dtype(dtype)
+    rng = np.random.default_rng(seed)
+    want = (rng.integers(-64, 65, (m, n, batch)) / 8.0).astype(np.float64)       # eighths: exact in fp16
+    want[want == 0] = 0.125
+    strideG = ldg * n + gap
+    got = np.full(strideG * batch, 777.0, dtype=npdt)
+    for b in range(batch):
+        got[b * strideG: b * strideG + ldg * n].reshape((ldg, n), order="F")[:m, :] = want[:, :, b].astype(npdt)
+    return want, got, ldg, strideG
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_comparator_reports_zero_on_an_exact_copy(dtype):
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    rel, ab = O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=1.0)
+    assert rel == 0.0 and ab == 0.0
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+@pytest.mark.parametrize("where", ["first", "last_of_batch0", "batch1", "last"])
+def test_comparator_finds_one_wrong_element_and_prices_it_exactly(dtype, where):
+    """One element off by delta (a power of two: exact in every dtype): abs = delta, rel = delta / max(|want|, floor),
+    wherever it sits -- first element, last element of a batch, inside batch >= 1 (strideG != ldg*n), the very last."""
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    i, j, b = {"first": (0, 0, 0), "last_of_batch0": (m - 1, n - 1, 0), "batch1": (3, 2, 1),
+               "last": (m - 1, n - 1, batch - 1)}[where]
+    delta = 0.5
+    got[b * strideG + j * ldg + i] += delta
+    w = abs(want[i, j, b])
+    for floor in (1e-30, 1.0, 100.0):
+        rel, ab = O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=floor)
+        assert ab == delta
+        assert rel == delta / max(w, floor)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_comparator_takes_the_maximum_not_the_last_or_the_sum(dtype):
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    got[0 * strideG + 1 * ldg + 2] += 0.25
+    got[1 * strideG + 4 * ldg + 6] -= 2.0           # the largest, in the middle of the buffer
+    got[2 * strideG + 0 * ldg + 0] += 0.125
+    rel, ab = O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=1e9)
+    assert ab == 2.0 and rel == 2.0 / 1e9
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+@pytest.mark.parametrize("bad", [np.nan, np.inf, -np.inf])
+def test_comparator_treats_nan_and_inf_in_the_result_as_unbounded_error(dtype, bad):
+    """An element the kernel never wrote stays NaN in the beta = 0 tests: it must not compare as 'no error'."""
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    got[2 * strideG + 3 * ldg + 4] = bad
+    rel, ab = O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=1.0)
+    assert rel == np.inf and ab == np.inf
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_comparator_ignores_padding_rows_and_batch_gaps(dtype):
+    """Rows m..ldg-1 and the elements between two batches are not part of the result (the padding check of the parity
+    tests is separate and bitwise); garbage there, NaN included, leaves the error at zero."""
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    for b in range(batch):
+        blk = got[b * strideG: b * strideG + ldg * n].reshape((ldg, n), order="F")
+        blk[m:, :] = np.nan
+        got[b * strideG + ldg * n: (b + 1) * strideG] = np.inf
+    rel, ab = O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=1.0)
+    assert rel == 0.0 and ab == 0.0
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, F64])
+def test_comparator_honours_the_leading_dimension_and_the_batch_stride(dtype):
+    """The same buffer read with a wrong ldg or strideG is a different matrix: the comparator must notice, i.e. it
+    really uses both (a comparator that assumed ldg = m or strideG = ldg*n would report zero on the right call only
+    by luck and a wrong figure here)."""
+    want, got, ldg, strideG = _cmp_case(dtype)
+    m, n, batch = want.shape
+    assert O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG, floor=1.0)[0] == 0.0
+    assert O.max_rel_err(dtype, got, ldg - 1, want, m, n, 1, strideG, floor=1.0)[0] > 0.0
+    assert O.max_rel_err(dtype, got, ldg, want, m, n, batch, strideG - 1, floor=1.0)[0] > 0.0
+    # a dense buffer compared as dense: ldg = m, strideG = m*n
+    dense = np.ascontiguousarray(want.reshape(-1, order="F").astype(O.np_dtype(dtype)))
+    assert O.max_rel_err(dtype, dense, m, want, m, n, batch, m * n, floor=1.0)[0] == 0.0
+
+
+def test_comparator_sees_every_element_of_a_large_result():
+    """The comparison runs threaded (a max-reduction over columns): an error in any column of a result large enough to
+    be split over all threads must come back, and the largest of many must win."""
+    m, n = 257, 1031
+    rng = np.random.default_rng(5)
+    want = rng.standard_normal((m, n))
+    got = want.astype(np.float32)
+    want = got.astype(np.float64)
+    for j in (0, 1, 515, 1029, 1030):
+        g = got.copy()
+        g[m - 1, j] += 4.0
+        rel, ab = O.max_rel_err(F32, np.ravel(g, order="F").copy(), m, want, m, n, floor=1e6)
+        assert abs(ab - 4.0) < 1e-5 and abs(rel - 4.0e-6) < 1e-11
+    g = got.copy()
+    g[:, ::7] += 1.0
+    g[100, 700] += 16.0
+    rel, ab = O.max_rel_err(F32, np.ravel(g, order="F").copy(), m, want, m, n, floor=1e6)
+    assert abs(ab - (17.0 if 700 % 7 == 0 else 16.0)) < 1e-4
+
+
+# ------------------------------------------------------------------ benchmark configuration 1 without a GPU
+
+def test_cfg1_inputs_native_cpu_gemm_against_fp64_oracle():
+    """SGEMM NN 1024^3, lda = ldb = ldc = 1024, A then B from one stream of seed 0, alpha = 1, beta = 0 over a poisoned
+    C: the native-precision CPU GEMM (fp32 chains, the timed CPU baseline) against the fp64 oracle within the
+    library's fp32 tolerance 1e-5 * sqrt(K).  This is the leg of the benchmark set that runs where no GPU is; the
+    GPU test of the same inputs is tests/test_gemm_gpu.py::test_cfg1_sgemm_nn_1024."""
+    import util as U
+    p = U.Problem(F32, 0, 0, 1024, 1024, 1024, 1.0, 0.0, seed=0, c_fill="nan")
+    assert np.array_equal(p.A, O.fill_uniform(1024 * 1024, F32, 0, 0))
+    assert np.array_equal(p.B, O.fill_uniform(1024 * 1024, F32, 0, 1024 * 1024))
+    got = p.C.copy()
+    O.gemm_native(F32, 0, 0, p.m, p.n, p.k, p.alpha, p.A, p.lda, p.B, p.ldb, p.beta, got, p.ldc)
+    assert np.all(np.isfinite(got))                     # beta = 0: the NaNs of the old C are gone
+    rel = U.check(p, got, "cfg1 on the CPU")
+    assert 0.0 < rel <= 1e-5 * np.sqrt(1024)
+    # a second opinion on a band of the result: numpy's float64 matmul of the same inputs
+    A = p.A.astype(np.float64).reshape((1024, 1024), order="F")
+    B = p.B.astype(np.float64).reshape((1024, 1024), order="F")
+    band = A[100:132, :] @ B
+    assert np.max(np.abs(p.exact()[100:132, :, 0] - band)) <= 1e-11
