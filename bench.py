@@ -5,8 +5,12 @@ carries the two HBM-bound skinny shapes (achieved algorithmic GB/s), three ragge
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
 A step is one GEMM launch through the C ABI on operands already resident in HBM.  Prints ONE JSON line.
-The timed region holds exactly K launches between two stream synchronisations; the per-launch duration
-used for the roofline comes from HIP events recorded on the same stream around the same K launches.
+After the W warm-up launches a settle phase keeps launching until the per-launch time has stopped drifting (the chip
+needs some tens of milliseconds of load to reach its steady clock and power state; the phase is reported as
+"settle_ms" / "settle_launches" and is not part of the timed region).  The timed region then holds exactly K launches
+between two stream synchronisations, cut into at least ten groups by HIP events recorded on the launch stream:
+"value" and "ms_per_step" are the MEDIAN per-launch time over the groups (the convention of this benchmark set: median
+of at least ten repetitions); mean, minimum and maximum over the groups and the wall-clock mean are reported beside it.
 """
 import argparse
 import json
@@ -19,14 +23,78 @@ sys.path.insert(0, ROOT)
 
 METRIC = "GEMM TFLOP/s + % of MFMA peak, fp16 & fp32 at 8192^3, 1 MI355X"
 PEAK_TFLOPS = {"f16": 2500.0, "f32": 157.3, "f64": 78.6}      # MI355X published dense matrix peaks
-# Bytes per launch that crossed the L2 <-> fabric boundary, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
-# this same command (each scaled by the counter's reading for a plain elementwise pass of known size; the
-# summaries with the commands are profiles/gemm_x16_f16_8192.txt and profiles/gemm_x16_f32_8192.txt).
-MEASURED_TRAFFIC_BYTES = {"f16": 1.626e9 + 0.135e9, "f32": 3.231e9 + 0.335e9}
+# Bytes per launch that crossed the L2 <-> fabric boundary come from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# same command (each scaled by the counter's reading for a plain elementwise pass of known size).  They are not measured
+# by this run: they are read from the "traffic:" line of the profile summary below, which names the kernel they were
+# taken on, and are reported only while that is still the kernel this run launches.
+TRAFFIC_PROFILE = {"f16": "profiles/gemm_x16_f16_8192.txt", "f32": "profiles/gemm_x16_f32_8192.txt"}
+
+
+def profiled_traffic(head, tile_config):
+    """(bytes per launch or None, where the figure comes from) from the profile summary's line
+       traffic: fetch_bytes=<float> write_bytes=<float> tile_config=<name> taken=<date>"""
+    import re
+    path = os.path.join(ROOT, TRAFFIC_PROFILE[head])
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, f"{TRAFFIC_PROFILE[head]} missing"
+    m = re.search(r"^traffic: fetch_bytes=(\S+) write_bytes=(\S+) tile_config=(\S+) taken=(\S+)", text, flags=re.M)
+    if not m:
+        return None, f"{TRAFFIC_PROFILE[head]} has no traffic line"
+    if m.group(3) != tile_config:
+        return None, f"{TRAFFIC_PROFILE[head]} was taken on {m.group(3)}, this run launches {tile_config}"
+    return float(m.group(1)) + float(m.group(2)), f"{TRAFFIC_PROFILE[head]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, taken {m.group(4)})"
+
+
+def timed_launches(torch, stream, step, steps, warmup, settle=True, groups=None):
+    """warm-up, settle phase, then exactly `steps` launches in event-delimited groups (one per launch up to 25 groups).
+    Returns a dict: median/mean/min/max per-launch ms over the groups, wall ms per launch, settle figures."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    settle_ms, settle_n = 0.0, 0
+    if settle:
+        # launch in chunks until >= 100 ms have passed and two consecutive chunks agree within 1.5 % (at most 600 ms)
+        t_begin = time.perf_counter()
+        prev = None
+        chunk = 4
+        while True:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            for _ in range(chunk):
+                step()
+            b.record(stream)
+            torch.cuda.synchronize()
+            cur = a.elapsed_time(b) / chunk
+            settle_n += chunk
+            settle_ms = (time.perf_counter() - t_begin) * 1e3
+            stable = prev is not None and abs(cur - prev) <= 0.015 * prev
+            if (settle_ms >= 100.0 and stable) or settle_ms >= 600.0:
+                break
+            prev = cur
+            if cur * chunk < 10.0:
+                chunk = min(chunk * 2, 4096)
+    groups = max(1, min(steps, groups or 25))
+    bounds = [round(i * steps / groups) for i in range(groups + 1)]
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(groups + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record(stream)
+    for g in range(groups):
+        for _ in range(bounds[g + 1] - bounds[g]):
+            step()
+        ev[g + 1].record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per = sorted(ev[g].elapsed_time(ev[g + 1]) / (bounds[g + 1] - bounds[g]) for g in range(groups))
+    med = per[len(per) // 2] if len(per) % 2 else 0.5 * (per[len(per) // 2 - 1] + per[len(per) // 2])
+    return {"median_ms": med, "mean_ms": ev[0].elapsed_time(ev[groups]) / steps, "min_ms": per[0], "max_ms": per[-1],
+            "wall_ms": wall_ms, "groups": groups, "settle_ms": settle_ms, "settle_launches": settle_n}
 
 
 def time_gemm(G, torch, dtype, m, n, k, steps, warmup, seed):
-    """Returns (wall ms per step, event ms per launch, config name, device tensors)."""
+    """Returns (timing dict of timed_launches, config description, device tensors)."""
     tdt = torch.float32 if dtype == G.F32 else torch.float16
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
@@ -47,19 +115,8 @@ def time_gemm(G, torch, dtype, m, n, k, steps, warmup, seed):
     def step():
         G.gemm(dtype, G.OP_N, G.OP_N, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(steps):
-        step()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    ev_ms = e0.elapsed_time(e1) / steps
-    return wall_ms, ev_ms, G.config_info(dtype, cid), (A, B, C)
+    t = timed_launches(torch, stream, step, steps, warmup)
+    return t, G.config_info(dtype, cid), (A, B, C)
 
 
 def spot_check(G, dtype, m, n, k, A, B, C):
@@ -96,16 +153,8 @@ def dgemm_legs(G, torch, steps, warmup):
         C = C0.clone()
         cid = G.select_config(G.F64, ta, tb, m, n, k, 1)
         nsteps = max(3, steps // 5) if tag == "8192" else steps
-        for _ in range(max(2, warmup // 4)):
-            G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(nsteps):
-            G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / nsteps
+        ms = timed_launches(torch, stream, lambda: G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream),
+                            nsteps, max(2, warmup // 4), settle=False)["median_ms"]
         # parity on a band of 64 rows of one fresh application (beta = 1 accumulates over the timed launches)
         C.copy_(C0)
         G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream)
@@ -144,16 +193,9 @@ def skinny_legs(G, torch, steps, warmup):
             B = (torch.rand(k * n, device="cuda", generator=gen) * 2 - 1).to(tdt)
             C = torch.empty(m * n, device="cuda", dtype=tdt)
             cid = G.select_config(dtype, 0, 0, m, n, k, 1)
-            for _ in range(warmup):
-                G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(steps):
-                G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream)
-            e1.record(stream)
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) / steps * 1e3
+            # small kernels: ten groups of at least twenty back-to-back launches each, median over the groups
+            us = timed_launches(torch, stream, lambda: G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream),
+                                max(steps, 200), max(warmup, 20), settle=False, groups=10)["median_ms"] * 1e3
             nbytes = (m * k + k * n + m * n) * esz
             out[f"{dname}_{m}x{n}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / us * 1e-3, 1),
                                             "frac_of_hbm_peak": round(nbytes / us * 1e-3 / 8000.0, 4),
@@ -181,16 +223,7 @@ def ragged_legs(G, torch, steps, warmup):
 
         def run():
             G.gemm(dtype, ta, tb, m, n, k, 1.0, A, lda, B, ldb, 0.0, C, m, G.CONFIG_AUTO, stream)
-        for _ in range(warmup):
-            run()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(steps):
-            run()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / steps * 1e3
+        us = timed_launches(torch, stream, run, max(steps, 20), max(warmup, 5), settle=False, groups=10)["median_ms"] * 1e3
         tf = 2.0 * m * n * k / us * 1e-6
         out[f"{dname}_{'NT'[ta]}{'NT'[tb]}_{m}x{n}x{k}"] = {"us": round(us, 1), "tflops": round(tf, 1),
                                                             "frac_of_peak": round(tf / PEAK_TFLOPS["f16" if dtype == G.F16 else "f32"], 4),
@@ -223,16 +256,8 @@ def config_legs(G, torch, steps, warmup):
         def run():
             G.gemm_strided_batched(dtype, ta, tb, m, n, k, alpha, A, lda, m * k, B, ldb, k * n, beta, C, m, m * n, batch,
                                    G.CONFIG_AUTO, stream)
-        for _ in range(warmup):
-            run()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(steps):
-            run()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        us = e0.elapsed_time(e1) / steps * 1e3
+        reps = max(steps, 20) if m >= 4096 else max(steps, 200)
+        us = timed_launches(torch, stream, run, reps, max(warmup, 10), settle=False, groups=10)["median_ms"] * 1e3
         tf = 2.0 * m * n * k * batch / us * 1e-6
         esz = 2 if dtype == G.F16 else 4
         gbps = batch * (m * k + k * n + m * n * (2 if beta != 0 else 1)) * esz / us * 1e-3
@@ -287,9 +312,9 @@ def main():
             continue
         steps = args.steps if name == "f16" else max(3, args.steps // 5)
         warm = args.warmup if name == "f16" else max(2, args.warmup // 5)
-        wall_ms, ev_ms, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, warm, seed=1234)
+        t, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, warm, seed=1234)
         rel, limit, host = spot_check(G, dtype, m, n, k, *tensors)
-        res[name] = dict(wall_ms=wall_ms, ev_ms=ev_ms, cfg=cfg, rel=rel, limit=limit, steps=steps)
+        res[name] = dict(t=t, wall_ms=t["wall_ms"], ev_ms=t["median_ms"], cfg=cfg, rel=rel, limit=limit, steps=steps)
         if name == "f16" and not args.no_cpu:
             res[name]["cpu"] = cpu_baseline(dtype, m, n, k, *host)
         del tensors, host
@@ -304,16 +329,9 @@ def main():
         C1 = torch.empty(m * n, device="cuda", dtype=torch.float16)
         st = torch.cuda.current_stream()
         cid1 = G.select_config(G.F16, 0, 0, m, n, k, 1)
-        for _ in range(20):
-            G.gemm(G.F16, G.OP_N, G.OP_N, m, n, k, 1.0, A1, m, B1, k, 0.0, C1, m, cid1, st)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(st)
-        for _ in range(50):
-            G.gemm(G.F16, G.OP_N, G.OP_N, m, n, k, 1.0, A1, m, B1, k, 0.0, C1, m, cid1, st)
-        e1.record(st)
-        torch.cuda.synchronize()
-        ones_tflops = flops / (e0.elapsed_time(e1) / 50) * 1e-9
+        t1 = timed_launches(torch, st, lambda: G.gemm(G.F16, G.OP_N, G.OP_N, m, n, k, 1.0, A1, m, B1, k, 0.0, C1, m, cid1, st),
+                            40, 10, settle=True)
+        ones_tflops = flops / t1["median_ms"] * 1e-9
         assert float(C1[12345]) == float(k)          # 8192 ones: exact in fp16
         del A1, B1, C1
         torch.cuda.empty_cache()
@@ -333,20 +351,28 @@ def main():
                 ceilings[f"{name}_{'random' if rnd else 'ones'}_operands"] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
     head = "f16" if "f16" in res else "f32"
     r = res[head]
-    tflops = flops / r["wall_ms"] * 1e-9
-    achieved = flops / r["ev_ms"] * 1e-9
+    t = r["t"]
+    tflops = flops / t["median_ms"] * 1e-9
+    achieved = tflops                               # the same K launches, timed by events on the launch stream
+    traffic, traffic_source = profiled_traffic(head, r["cfg"]["name"])
     alg_bytes = (m * k + k * n + m * n) * (2 if head == "f16" else 4)
     out = {
         "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": r["steps"],
-        "warmup": args.warmup, "ms_per_step": round(r["wall_ms"], 4), "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "ms_per_step": round(t["median_ms"], 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": head, "data": "synthetic",
         "config": {"workload": f"{'H' if head == 'f16' else 'S'}GEMM NN M=N=K=8192 lda=ldb=ldc=8192 alpha=1 beta=0, "
                                + ("A,B ~ N(0,1)*0.1 rounded to fp16, fp32 accumulate" if head == "f16" else "A,B ~ U[-1,1]"),
                    "tile_config": r["cfg"]["name"]},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[head], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS[head], 4), "traffic": MEASURED_TRAFFIC_BYTES[head],
+                     "frac": round(achieved / PEAK_TFLOPS[head], 4), "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes": alg_bytes, "flops_per_launch": flops,
-                     "kernel_ms": round(r["ev_ms"], 4)},
+                     "kernel_ms": round(t["median_ms"], 4)},
+        "timing": {"statistic": "median over the groups of the timed region; value and ms_per_step use it",
+                   "groups": t["groups"], "median_ms": round(t["median_ms"], 4), "mean_ms": round(t["mean_ms"], 4),
+                   "min_ms": round(t["min_ms"], 4), "max_ms": round(t["max_ms"], 4),
+                   "wall_ms_per_step": round(t["wall_ms"], 4), "settle_ms": round(t["settle_ms"], 1),
+                   "settle_launches": t["settle_launches"],
+                   "mean_tflops": round(flops / t["mean_ms"] * 1e-9, 2), "best_tflops": round(flops / t["min_ms"] * 1e-9, 2)},
         "max_rel_err": float(f"{r['rel']:.3e}"), "rel_err_limit": float(f"{r['limit']:.3e}"),
         "parity_ok": bool(r["rel"] <= r["limit"]),
     }
@@ -360,7 +386,7 @@ def main():
             out["roofline"]["frac_of_measured_mfma_ceiling"] = round(achieved / c["tflops"], 4)
     if head == "f16" and "f32" in res:
         q = res["f32"]
-        out["also"] = {"fp32_tflops": round(flops / q["wall_ms"] * 1e-9, 2), "fp32_ms_per_step": round(q["wall_ms"], 4),
+        out["also"] = {"fp32_tflops": round(flops / q["ev_ms"] * 1e-9, 2), "fp32_ms_per_step": round(q["ev_ms"], 4),
                        "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
                        "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
                        "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}

@@ -30,7 +30,7 @@ FLAGS = [
 
 
 def _units():
-    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("probe.hip", "probe.o", []), ("inst_ring_wide.hip", "inst_ring_wide.o", [])]
+    units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("probe.hip", "probe.o", [])]
     for dtype in (0, 1):
         for tile in range(NUM_TILES):
             units.append(("inst_staged.hip", f"inst_staged_{dtype}_{tile}.o",

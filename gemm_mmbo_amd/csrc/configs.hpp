@@ -65,7 +65,7 @@ constexpr int ring_bk(int dtype) { return dtype == 0 ? 16 : 32; }
 
 // Tiles of the 16x16-block ring kernel with accumulation-register accumulators (gemm_x16.hpp), both element types;
 // depthU is 32 (fp16) / 16 (fp32).
-// Config ids continue after the ring and wide ones:  x16_tile + NUM_X16_TILES * split_index.
+// Config ids continue after the ring ones:  x16_tile + NUM_X16_TILES * split_index.
 constexpr int NUM_X16_TILES = 5;
 constexpr RingRow kX16Tiles[NUM_X16_TILES] = {
     {256, 256, 2, 2, 5},     // four wavefronts of 128 x 128: 256 accumulator registers per lane, one work-group per CU
@@ -74,5 +74,22 @@ constexpr RingRow kX16Tiles[NUM_X16_TILES] = {
     {128,  64, 2, 2, 6},     //  72 KB, two per CU
     { 64,  64, 2, 2, 6},     //  48 KB, three per CU
 };
+
+// Config ids (fp32 and fp16 share them): [0, kStagedConfigs) the staged kernel's (tile, split) pairs, then the ring
+// kernel's (ring tile, split) pairs, then the x16 kernel's.  split_index indexes kSplits.
+constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
+constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
+constexpr int kX16Base = kStagedConfigs + kRingConfigs;
+constexpr int kX16Configs = NUM_X16_TILES * NUM_SPLITS;
+constexpr int kNumConfigs = kX16Base + kX16Configs;
+constexpr int split_index(int split)
+{
+    for (int i = 0; i < NUM_SPLITS; ++i)
+        if (kSplits[i] == split) return i;
+    return -1;
+}
+constexpr int staged_config_id(int tile, int split_idx) { return tile + NUM_TILES * split_idx; }
+constexpr int ring_config_id(int tile, int split_idx) { return kStagedConfigs + tile + NUM_RING_TILES * split_idx; }
+constexpr int x16_config_id(int tile, int split_idx) { return kX16Base + tile + NUM_X16_TILES * split_idx; }
 
 }  // namespace mmbo

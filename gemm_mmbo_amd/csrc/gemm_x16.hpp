@@ -730,7 +730,10 @@ gemm_x16_kernel(const GemmArgs args)
         static_for<FM * FN>([&](auto IJ) {
             constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
             float *p = ws + (size_t)(wcol0 + j * 16) * args.m + wrow0 + i * 16;
-            *reinterpret_cast<f32x4 *>(p) = f32x4{acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
+            // with m not a multiple of four the columns of the workspace start at any multiple of four bytes: the vector
+            // type only promises that much alignment (the hardware takes a 16-byte store at any dword)
+            typedef f32x4 __attribute__((aligned(4))) f32x4_dword_aligned;
+            *reinterpret_cast<f32x4_dword_aligned *>(p) = f32x4{acc_read<base>(), acc_read<base + 1>(), acc_read<base + 2>(), acc_read<base + 3>()};
         });
         continue;
     }

@@ -28,9 +28,6 @@ int staged_lds_bytes();
 template <int DTYPE, int TILE>
 hipError_t launch_ring(int transA, int transB, const GemmArgs &args, hipStream_t stream);
 
-// HGEMM 256 x 256 ring kernel with 64-k units for the k-contiguous operand; NN and TT only, k % 64 == 0, k >= 512.
-hipError_t launch_hgemm_ring_wide(int transA, int transB, const GemmArgs &args, hipStream_t stream);
-
 // 16x16-block ring kernel (gemm_x16.hpp) of x16 tile row TILE; grid = (nwg0*nwg1, 1, batch*splits).
 template <int DTYPE, int TILE>
 hipError_t launch_x16(int transA, int transB, const GemmArgs &args, hipStream_t stream);

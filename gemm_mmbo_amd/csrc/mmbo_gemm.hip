@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "configs.hpp"
 #include "gemm_common.hpp"
@@ -18,18 +19,11 @@ namespace mmbo {
 
 namespace {
 
-// Config ids: [0, kStagedConfigs) are the staged kernel's (tile, split) pairs, then the ring kernel's
-// (ring tile, split) pairs.  A ring config applies when m, n are multiples of its tile, k splits into whole
-// slices and A, B are 16-byte aligned; otherwise the call is refused with MMBO_ERR_INVALID_CONFIG.
-constexpr int kStagedConfigs = NUM_TILES * NUM_SPLITS;
-constexpr int kRingConfigs = NUM_RING_TILES * NUM_SPLITS;
-constexpr int kWideConfig = kStagedConfigs + kRingConfigs;      // HGEMM NN/TT 256x256 ring with 64-k units
-constexpr int kX16Base = kWideConfig + 1;                      // ring on 16x16 MFMA blocks, (x16 tile, split) pairs
-constexpr int kX16Configs = NUM_X16_TILES * NUM_SPLITS;
-constexpr int kNumConfigs = kX16Base + kX16Configs;
-
+// Config ids (configs.hpp): [0, kStagedConfigs) are the staged kernel's (tile, split) pairs, then the ring kernel's
+// (ring tile, split) pairs, then the x16 kernel's.  A ring config applies when m, n are multiples of its tile, k splits
+// into whole slices and A, B are 16-byte aligned; otherwise the call is refused with MMBO_ERR_INVALID_CONFIG.
 struct ConfigRef {
-    bool ring;      // a whole-tile kernel (ring, wide or x16): no edge handling
+    bool ring;      // a direct-to-LDS kernel (ring or x16)
     int tile;
     int split;
     bool x16;
@@ -37,19 +31,11 @@ struct ConfigRef {
 inline ConfigRef config_ref(int id)
 {
     if (id >= kX16Base) return {true, (id - kX16Base) % NUM_X16_TILES, kSplits[(id - kX16Base) / NUM_X16_TILES], true};
-    if (id == kWideConfig) return {true, 0, 1, false};          // same tile and grid as ring tile 0, no split
     if (id < kStagedConfigs) return {false, id % NUM_TILES, kSplits[id / NUM_TILES], false};
     id -= kStagedConfigs;
     return {true, id % NUM_RING_TILES, kSplits[id / NUM_RING_TILES], false};
 }
-inline int x16_config_id(int tile, int split_index) { return kX16Base + tile + NUM_X16_TILES * split_index; }
 inline bool valid_dtype(int dtype) { return dtype == MMBO_F32 || dtype == MMBO_F16 || dtype == MMBO_F64; }
-inline int ring_config_id(int tile, int split_index) { return kStagedConfigs + tile + NUM_RING_TILES * split_index; }
-
-inline bool wide_ok(int dtype, int transA, int transB, size_t m, size_t n, size_t k)
-{
-    return dtype == MMBO_F16 && transA == transB && m % 256 == 0 && n % 256 == 0 && k % 64 == 0 && k >= 512;
-}
 
 // Does the ring (x16 = false) or x16 config (tile, split) take this shape?  Ring: m, n whole tiles, k whole slices, the
 // same number for every split; A and B 16-byte aligned (checked at the call).  x16: any shape and alignment (its loads
@@ -77,41 +63,61 @@ int hip_fail(hipError_t e)
     return MMBO_ERR_HIP;
 }
 
-// ---- split-K workspace: one grow-only buffer per device ---------------------------------------
+// ---- split-K workspace ------------------------------------------------------------------------
+// A workspace holds the partial sums of one GEMM with GlobalSplitU > 1: [split][batch][n][m] fp32.
 constexpr int kMaxDevices = 64;
-std::mutex g_ws_mutex;
-float *g_ws[kMaxDevices] = {};
-size_t g_ws_bytes[kMaxDevices] = {};
 
-int workspace(size_t bytes, float **out)
+// Library-owned workspaces: one per (device, stream), so GEMMs on different streams never share partial sums, grown on
+// demand.  Only launches on that stream ever touch a slot's buffer, so growing it waits for that stream alone.  The
+// mutex is held from the lookup until the launches that use the buffer have been queued: another host thread that
+// grows (frees) the same stream's buffer then does so after them in stream order.
+struct WsSlot {
+    hipStream_t stream;
+    char *base;
+    size_t bytes;
+};
+std::mutex g_ws_mutex;
+std::vector<WsSlot> g_ws_slots[kMaxDevices];
+
+// The buffer of (current device, stream), at least `bytes` large.  Caller holds g_ws_mutex.
+int workspace(hipStream_t stream, size_t bytes, char **out)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e);
     if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (g_ws_bytes[dev] < bytes) {
-        if (g_ws[dev]) {
-            // earlier launches may still be reading the old buffer
-            e = hipDeviceSynchronize();
+    std::vector<WsSlot> &slots = g_ws_slots[dev];
+    WsSlot *slot = nullptr;
+    for (WsSlot &sl : slots)
+        if (sl.stream == stream) slot = &sl;
+    if (!slot) {
+        slots.push_back(WsSlot{stream, nullptr, 0});
+        slot = &slots.back();
+    }
+    if (slot->bytes < bytes) {
+        if (slot->base) {
+            // earlier launches on this stream may still be using the old buffer (fails under stream capture: a captured
+            // call must find its workspace already large enough, or use the entry point that allocates nothing)
+            e = hipStreamSynchronize(stream);
             if (e != hipSuccess) return hip_fail(e);
-            (void)hipFree(g_ws[dev]);
-            g_ws[dev] = nullptr;
-            g_ws_bytes[dev] = 0;
+            (void)hipFree(slot->base);
+            slot->base = nullptr;
+            slot->bytes = 0;
         }
         size_t want = bytes + bytes / 4;
-        if (hipMalloc(reinterpret_cast<void **>(&g_ws[dev]), want) != hipSuccess) {
+        void *p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) {
             (void)hipGetLastError();
-            if (hipMalloc(reinterpret_cast<void **>(&g_ws[dev]), bytes) != hipSuccess) {
+            want = bytes;
+            if (hipMalloc(&p, want) != hipSuccess) {
                 (void)hipGetLastError();
-                g_ws[dev] = nullptr;
                 return MMBO_ERR_WORKSPACE;
             }
-            want = bytes;
         }
-        g_ws_bytes[dev] = want;
+        slot->base = static_cast<char *>(p);
+        slot->bytes = want;
     }
-    *out = g_ws[dev];
+    *out = slot->base;
     return MMBO_OK;
 }
 
@@ -293,12 +299,6 @@ int mmbo_config_info(int dtype, int config_id, mmbo_config_desc *out)
         return MMBO_OK;
     }
     const ConfigRef c = config_ref(config_id);
-    if (config_id == kWideConfig) {
-        std::snprintf(out->name, sizeof(out->name), "MT256x256x64_WT064x128_W8_GSU01_DTL1_RING4+3U");
-        out->macro_tile_m = 256; out->macro_tile_n = 256; out->depth_u = 64; out->threads = 512;
-        out->wave_tile_m = 64; out->wave_tile_n = 128; out->split_k = 1; out->lds_bytes = 160 * 1024;
-        return MMBO_OK;
-    }
     if (c.ring) {
         const RingRow &r = c.x16 ? kX16Tiles[c.tile] : kRingTiles[c.tile];
         std::snprintf(out->name, sizeof(out->name), "MT%03dx%03dx%02d_WT%03dx%03d_W%d_GSU%02d_DTL1_RING%d%s", r.bm, r.bn,
@@ -414,11 +414,11 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
     if ((transA | transB) & ~1) return -MMBO_ERR_INVALID_OP;
     if (batch < 0) return -MMBO_ERR_INVALID_SIZE;
     if (m == 0 || n == 0 || batch == 0) return 0;
+    for (const TunedRow &t : kTuned)
+        if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
+            t.batch == batch)
+            return t.config_id;
     if (dtype == MMBO_F64) {
-        for (const TunedRow &t : kTuned)
-            if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
-                t.batch == batch)
-                return t.config_id;
         int best = 0;
         double best_t = 0.0;
         for (int tile = 0; tile < NUM_F64_TILES; ++tile) {
@@ -427,10 +427,6 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
         }
         return best;
     }
-    for (const TunedRow &t : kTuned)
-        if (t.dtype == dtype && t.transA == transA && t.transB == transB && t.m == m && t.n == n && t.k == k &&
-            t.batch == batch)
-            return t.config_id;
     // Whole-tile kernels (deeper prefetch, no edge handling) measured faster than the staged kernel on every shape
     // they apply to: where one applies, the fastest of them by model_time_ring takes the call.  fp16: the x16 family
     // (16x16x32 MFMAs), except that the 64 x 64 tile is faster on 32x32x16; fp32: the ring family, except that the
@@ -513,21 +509,29 @@ int mmbo_release_workspace(void)
     if (e != hipSuccess) return hip_fail(e);
     if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (g_ws[dev]) {
+    if (!g_ws_slots[dev].empty()) {
         e = hipDeviceSynchronize();
         if (e != hipSuccess) return hip_fail(e);
-        e = hipFree(g_ws[dev]);
-        g_ws[dev] = nullptr;
-        g_ws_bytes[dev] = 0;
-        if (e != hipSuccess) return hip_fail(e);
+        hipError_t first = hipSuccess;
+        for (WsSlot &sl : g_ws_slots[dev])
+            if (sl.base) {
+                e = hipFree(sl.base);
+                if (e != hipSuccess && first == hipSuccess) first = e;
+            }
+        g_ws_slots[dev].clear();
+        if (first != hipSuccess) return hip_fail(first);
     }
     return MMBO_OK;
 }
 
-int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
-                              const void *alpha, const void *A, size_t lda, long long strideA,
-                              const void *B, size_t ldb, long long strideB, const void *beta, void *C,
-                              size_t ldc, long long strideC, int batch, int config_id, void *stream)
+}  // extern "C"
+
+namespace {
+
+int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+              const void *alpha, const void *A, size_t lda, long long strideA,
+              const void *B, size_t ldb, long long strideB, const void *beta, void *C,
+              size_t ldc, long long strideC, int batch, int config_id, void *stream)
 {
     if (!valid_dtype(dtype)) return MMBO_ERR_INVALID_DTYPE;
     if ((transA & ~1) || (transB & ~1)) return MMBO_ERR_INVALID_OP;
@@ -571,8 +575,7 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
                     static const int x16_of_ring[NUM_RING_TILES] = {0, 2, 3, 4};
                     int si = 0;
                     while (si + 1 < NUM_SPLITS && kSplits[si] != c.split) ++si;
-                    const bool wide_pick = config_id == kWideConfig;
-                    const int tile = wide_pick ? 0 : x16_of_ring[c.tile];
+                    const int tile = x16_of_ring[c.tile];
                     config_id = ring_shape_ok(dtype, tile, c.split, transA, transB, m, n, k, true)
                                     ? x16_config_id(tile, si) : select_staged(dtype, m, n, k, batch);
                 }
@@ -593,8 +596,6 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
     const RingRow &rr = cref.x16 ? kX16Tiles[cref.tile] : kRingTiles[cref.ring ? cref.tile : 0];
     TileRow r = f64 ? kTilesF64[config_id] : cref.ring ? TileRow{rr.bm, rr.bn, ring_bk(dtype), 0, 0} : tile_row(dtype, cref.tile);
     if (cref.ring && !ring_shape_ok(dtype, cref.tile, split, transA, transB, m, n, k, cref.x16)) return MMBO_ERR_INVALID_CONFIG;
-    const bool wide = !f64 && config_id == kWideConfig;
-    if (wide && !wide_ok(dtype, transA, transB, m, n, k)) return MMBO_ERR_INVALID_CONFIG;
 
     if (!tile_span_ok(r, transA, transB, lda, ldb, esz)) return MMBO_ERR_INVALID_CONFIG;
 
@@ -634,14 +635,20 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
+    // Split-K: the partial sums go to the stream's own workspace, and both launches that use it (the
+    // GEMM and the reduction, which adds the splits in ascending order) are queued before the lock on the workspace
+    // table is given up.
+    std::unique_lock<std::mutex> ws_lock;
     if (split > 1) {
-        size_t bytes = (size_t)split * batch * m * n * sizeof(float);
-        int rc = workspace(bytes, &a.ws);
+        const size_t bytes = (size_t)split * batch * m * n * sizeof(float);
+        char *base = nullptr;
+        ws_lock = std::unique_lock<std::mutex>(g_ws_mutex);
+        int rc = workspace(s, bytes, &base);
         if (rc != MMBO_OK) return rc;
+        a.ws = reinterpret_cast<float *>(base);
     }
     hipError_t e;
     if (f64) e = dispatch_dgemm<0>(cref.tile, transA, transB, a, s);
-    else if (wide) e = launch_hgemm_ring_wide(transA, transB, a, s);
     else if (cref.x16) e = dtype == MMBO_F32 ? dispatch_x16<0, 0>(cref.tile, transA, transB, a, s)
                                         : dispatch_x16<1, 0>(cref.tile, transA, transB, a, s);
     else if (cref.ring) e = dtype == MMBO_F32 ? dispatch_ring<0, 0>(cref.tile, transA, transB, a, s)
@@ -654,6 +661,19 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
         if (e != hipSuccess) return hip_fail(e);
     }
     return MMBO_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+                              const void *alpha, const void *A, size_t lda, long long strideA,
+                              const void *B, size_t ldb, long long strideB, const void *beta, void *C,
+                              size_t ldc, long long strideC, int batch, int config_id, void *stream)
+{
+    return gemm_impl(dtype, transA, transB, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch,
+                     config_id, stream);
 }
 
 int mmbo_gemm(int dtype, int transA, int transB, size_t m, size_t n, size_t k, const void *alpha,

@@ -6,6 +6,8 @@
 
 #include <cstddef>
 
+#include "configs.hpp"
+
 namespace mmbo {
 
 struct TunedRow {
@@ -16,27 +18,35 @@ struct TunedRow {
     float tflops;     // measured with that config, for the record
 };
 
+// Ring tiles (kRingTiles): 0 = 256x256, 1 = 128x128, 2 = 128x64, 3 = 64x64; x16 tiles (kX16Tiles): 0 = 256x256 on four
+// wavefronts, 1 = on eight, 2 = 128x128, 3 = 128x64, 4 = 64x64.  The ids are built from (tile, GlobalSplitU), so a row
+// keeps its meaning when a tile or a split factor is added to the tables.
+constexpr int ring_id(int tile, int split) { return ring_config_id(tile, split_index(split)); }
+constexpr int x16_id(int tile, int split) { return x16_config_id(tile, split_index(split)); }
+
 constexpr TunedRow kTuned[] = {
     //dtype ta tb m n k batch id TFLOP/s
-    {0, 0, 0, 1024, 1024, 1024, 1, 33, 93.0f},
-    {0, 0, 1, 4096, 4096, 4096, 1, 30, 140.2f},
-    {0, 1, 0, 4096, 4096, 4096, 1, 51, 145.0f},
-    {0, 0, 0, 1023, 777, 513, 1, 55, 46.6f},
-    {1, 0, 0, 1023, 777, 513, 1, 55, 82.4f},
-    {0, 0, 0, 4096, 128, 4096, 1, 41, 95.0f},
-    {1, 0, 0, 4096, 128, 4096, 1, 37, 272.2f},
-    {0, 0, 0, 128, 4096, 8192, 1, 45, 108.8f},
-    {1, 0, 0, 128, 4096, 8192, 1, 40, 423.9f},
-    {1, 1, 0, 512, 512, 512, 64, 51, 442.8f},
-    {0, 0, 0, 2048, 2048, 2048, 1, 33, 117.5f},
-    {1, 0, 0, 2048, 2048, 2048, 1, 53, 761.2f},
-    {0, 0, 1, 44160, 2048, 384, 1, 53, 120.5f},
-    {0, 0, 0, 8192, 8192, 8192, 1, 51, 145.3f},
-    {1, 0, 0, 8192, 8192, 8192, 1, 51, 1330.0f},
-    {0, 0, 0, 4096, 4096, 4096, 1, 51, 143.6f},
-    {1, 0, 0, 4096, 4096, 4096, 1, 51, 1245.0f},
-    {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // the reference's HPL trailing update (src/gemm/run.sh:2-5)
+    {0, 0, 0, 1024, 1024, 1024, 1, ring_id(3, 1), 93.0f},
+    {0, 0, 1, 4096, 4096, 4096, 1, ring_id(0, 1), 140.2f},
+    {0, 1, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 145.0f},
+    {0, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 46.6f},
+    {1, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 82.4f},
+    {0, 0, 0, 4096, 128, 4096, 1, ring_id(3, 4), 95.0f},
+    {1, 0, 0, 4096, 128, 4096, 1, ring_id(3, 2), 272.2f},
+    {0, 0, 0, 128, 4096, 8192, 1, ring_id(3, 8), 108.8f},
+    {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 423.9f},
+    {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 442.8f},
+    {0, 0, 0, 2048, 2048, 2048, 1, ring_id(3, 1), 117.5f},
+    {1, 0, 0, 2048, 2048, 2048, 1, x16_id(2, 1), 761.2f},
+    {0, 0, 1, 44160, 2048, 384, 1, x16_id(2, 1), 120.5f},
+    {0, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 145.3f},
+    {1, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 1330.0f},
+    {0, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 143.6f},
+    {1, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 1245.0f},
+    {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // fp64 ids are rows of kTilesF64; the reference's HPL trailing update (src/gemm/run.sh:2-5)
     {2, 0, 0, 8192, 8192, 8192, 1, 0, 69.7f},
 };
+static_assert(ring_id(3, 1) == 33 && ring_id(3, 2) == 37 && x16_id(0, 1) == 50 && x16_id(4, 16) == 74,
+              "config id layout: 30 staged ids, 20 ring ids, 25 x16 ids");
 
 }  // namespace mmbo

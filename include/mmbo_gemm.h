@@ -20,8 +20,9 @@
  *     MMBO_F64: double A, B, C, alpha, beta (the reference's own element type); fp64 MFMA accumulate;
  *   - the launch is asynchronous on `stream` (a hipStream_t, NULL = the null stream the
  *     reference uses, src/gemm/common.h:12); the caller synchronises.  Configs with GlobalSplitU > 1 keep their
- *     partial sums in one workspace per device: two such GEMMs must not be in flight on different streams of
- *     one device at the same time (the same stream, or configs without split-K, are fine);
+ *     partial sums in a workspace the library owns, one per (device, stream): GEMMs on different streams never
+ *     share one, and calls from several host threads are safe.  A workspace is allocated on the first split-K call
+ *     on its stream and grown when a call needs more (this waits for that stream's earlier work);
  *   - config_id selects a row of the tile-config table, like the reference's kernelId
  *     (src/gemm/constants.h:34-47,106-135); MMBO_CONFIG_AUTO lets the per-shape table pick.  Every shape runs
  *     under MMBO_CONFIG_AUTO.  Named configs: the general kernel's (no "DTL1" in the name) take any shape and
@@ -130,8 +131,9 @@ int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsi
  * L2.  A bijection of [0, tiles*batch); needs batch % 8 == 0.  Pure host logic. */
 int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, unsigned *tile, unsigned *batch_index);
 
-/* Release the split-K workspace held for the current device (allocated lazily, grown on
- * demand, reused across calls).  The reference never frees what it loads (src/gemm/driver.h:41). */
+/* Release the split-K workspaces held for the current device (one per stream that ran a split-K config; allocated
+ * lazily, grown on demand, reused across calls).  Waits for the device.  The reference never frees what it loads
+ * (src/gemm/driver.h:41). */
 int mmbo_release_workspace(void);
 
 /* Measures what the MFMA pipes of the current device sustain with nothing else running: a register-only loop

@@ -80,20 +80,19 @@ def test_batches_of_small_problems_one_per_xcd():
             d = G.config_info(dtype, cid)
             name = d["name"]
             ring_only = "DTL1" in name and "_ACC" not in name
-            if "GSU01" not in name or ("+3U" in name and dtype != F16):
+            if "GSU01" not in name:
                 continue
             bm, bn = d["macro_tile_m"], d["macro_tile_n"]
-            bk = 64 if "+3U" in name else d["depth_u"]
+            bk = d["depth_u"]
             shapes = [(bm, bn, 4 * bk, 8), (2 * bm, 2 * bn, 2 * bk, 16), (4 * bm, 8 * bn, 2 * bk, 8)]
             if not ring_only and bm <= 128:
                 shapes.append((2 * bm - 3, 3 * bn - 5, 3 * bk + 1, 24))
             for (m, n, k, batch) in shapes:
                 if m * n * batch > 48 << 20:
                     continue
-                ta, tb = (cid % 2, (cid // 2) % 2) if "+3U" not in name else (0, 0)
-                k = max(k, 512) if "+3U" in name else k             # the wide-unit kernel needs k >= 512
+                ta, tb = cid % 2, (cid // 2) % 2
                 (ar, ac), (br, bc) = U.stored_shape(ta, m, k), U.stored_shape(tb, k, n)
-                gap = 0 if "+3U" in name else 8
+                gap = 8
                 p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.5, batch=batch, seed=40 + cid, dist=dist, c_fill="uniform",
                               strides=(ar * ac + gap, br * bc + gap, m * n + gap))
                 _run_and_check(p, cid, label=f"{name} {m}x{n}x{k} b{batch}")
@@ -136,11 +135,6 @@ def test_every_config_aligned_interior(dtype):
     import gemm_mmbo_amd as G
     for cid in range(G.num_configs(dtype)):
         p = U.Problem(dtype, 0, 0, 512, 512, 1024, 1.0, 0.0, seed=50 + cid, c_fill="nan")
-        name = G.config_info(dtype, cid)["name"]
-        if dtype == F32 and "+3U" in name:      # an fp16-only kernel
-            with pytest.raises(G.MmboError):
-                U.run_gpu(p, cid)
-            continue
         _run_and_check(p, cid, label=f"config {cid}")
 
 
@@ -148,7 +142,7 @@ def _ring_ids(dtype):
     """Config ids of the generic direct-to-LDS ring kernel (32x32 MFMA blocks)."""
     import gemm_mmbo_amd as G
     names = {c: G.config_info(dtype, c)["name"] for c in range(G.num_configs(dtype))}
-    return [c for c, nm in names.items() if "DTL1" in nm and "+3U" not in nm and "_ACC" not in nm]
+    return [c for c, nm in names.items() if "DTL1" in nm and "_ACC" not in nm]
 
 
 def _x16_ids(dtype=F16):
@@ -156,31 +150,6 @@ def _x16_ids(dtype=F16):
     import gemm_mmbo_amd as G
     mark = "MFMA16x16x32_ACC" if dtype == F16 else "MFMA16x16x4_ACC"
     return [c for c in range(G.num_configs(dtype)) if mark in G.config_info(dtype, c)["name"]]
-
-
-def _wide_id():
-    import gemm_mmbo_amd as G
-    (cid,) = [c for c in range(G.num_configs(F16)) if "+3U" in G.config_info(F16, c)["name"]]
-    return cid
-
-
-def test_wide_unit_ring_kernel_nn_tt():
-    """The HGEMM NN/TT variant that fetches the k-contiguous operand in 64-k units: K from the
-    shortest it takes (512) up, unit counts that are and are not multiples of the three unit buffers, beta, batches;
-    refused for NT/TN, fp32, short or odd K."""
-    import gemm_mmbo_amd as G
-    cid = _wide_id()
-    for (ta, tb) in ((0, 0), (1, 1)):
-        for (m, n, k, alpha, beta, batch) in ((256, 256, 512, 1.0, 0.0, 1), (512, 256, 576, 1.5, 0.5, 1), (256, 768, 1024, -1.0, 1.0, 2),
-                                              (768, 512, 4096, 1.0, 0.0, 1), (256, 256, 640, 1.0, 0.0, 1), (256, 512, 704, 1.0, 1.0, 1)):
-            p = U.Problem(F16, ta, tb, m, n, k, alpha, beta, batch=batch, seed=90 + k, dist="normal",
-                          c_fill="uniform" if beta else "nan")
-            _run_and_check(p, cid, label=f"wide {m}x{n}x{k}")
-    for (dtype, ta, tb, k) in ((F16, 0, 1, 1024), (F16, 1, 0, 1024), (F32, 0, 0, 1024), (F16, 0, 0, 448), (F16, 0, 0, 1056)):
-        p = U.Problem(dtype, ta, tb, 256, 256, k, 1.0, 0.0, seed=3, c_fill="nan")
-        with pytest.raises(G.MmboError) as e:
-            U.run_gpu(p, cid)
-        assert e.value.status == 5
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -467,6 +436,87 @@ def test_repeatable_bitwise_including_split_k():
             a, _ = U.run_gpu(p, cid)
             b, _ = U.run_gpu(p, cid)
             assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+
+
+def test_split_k_every_family_ragged_and_batched():
+    """GlobalSplitU > 1 in every kernel family: whole tiles, edge tiles with m % 4 != 0 (the partial sums are then stored
+    and added element by element) and with m % 4 == 0, uneven splits of k, batches, beta; one call after the other on
+    one stream, so on one workspace."""
+    import gemm_mmbo_amd as G
+    ran = 0
+    for dtype in (F32, F16):
+        for cid in range(G.num_configs(dtype)):
+            d = G.config_info(dtype, cid)
+            name, sp, bm, bn, bk = d["name"], d["split_k"], d["macro_tile_m"], d["macro_tile_n"], d["depth_u"]
+            if sp == 1 or bm > 128 and sp > 4:
+                continue
+            ring_only = "DTL1" in name and "_ACC" not in name
+            ta, tb = cid % 2, (cid // 2) % 2
+            cases = [(ta, tb, 2 * bm, 3 * bn, sp * 3 * bk, 1.0, 0.0, 1, 0), (tb, ta, bm, 2 * bn, sp * 2 * bk, -1.5, 0.5, 3, 4)]
+            if not ring_only:
+                cases += [(ta, tb, 2 * bm - 3, bn + 5, sp * 2 * bk + bk + 7, 1.0, 0.0, 1, 1),
+                          (1, 0, bm + 12, 2 * bn - 1, sp * 4 * bk - 3, 0.5, 1.0, 2, 0)]
+            for (a, b, m, n, k, alpha, beta, batch, pad) in cases:
+                p = U.Problem(dtype, a, b, m, n, k, alpha, beta, ldc=m + pad, batch=batch, seed=70 + cid,
+                              dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
+                _run_and_check(p, cid, label=f"config {cid} {name} {m}x{n}x{k} b{batch}")
+                ran += 1
+    assert ran >= 100
+
+
+def test_split_k_on_two_streams_at_the_same_time():
+    """Every stream has its own split-K workspace: GEMMs with GlobalSplitU > 1 queued on two streams without any
+    synchronisation between them (the reference's launcher is not re-entrant at all, src/gemm/driver.h:41)."""
+    import torch
+    import gemm_mmbo_amd as G
+    probs = [U.Problem(F16, 0, 0, 4096, 128, 4096, 1.0, 0.0, seed=81, c_fill="nan"),
+             U.Problem(F32, 0, 0, 128, 4096, 2048, 1.0, 0.5, seed=82, c_fill="uniform")]
+    cids = [G.select_config(p.dtype, 0, 0, p.m, p.n, p.k) for p in probs]
+    for p, cid in zip(probs, cids):
+        assert G.config_info(p.dtype, cid)["split_k"] > 1
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    tdt = {F32: torch.float32, F16: torch.float16}
+    dev = [[torch.from_numpy(x).cuda() for x in (p.A, p.B, p.C)] for p in probs]
+    outs = [[torch.empty_like(d[2]) for _ in range(6)] for d in dev]
+    torch.cuda.synchronize()
+    for rep in range(6):
+        for i, (p, cid) in enumerate(zip(probs, cids)):
+            with torch.cuda.stream(streams[i]):
+                outs[i][rep].copy_(dev[i][2], non_blocking=True)
+                G.gemm(p.dtype, 0, 0, p.m, p.n, p.k, p.alpha, dev[i][0], p.lda, dev[i][1], p.ldb, p.beta, outs[i][rep], p.ldc,
+                       cid, streams[i])
+    torch.cuda.synchronize()
+    for i, p in enumerate(probs):
+        first = outs[i][0].cpu().numpy()
+        U.check(p, first, f"stream {i}")
+        for rep in range(1, 6):
+            assert np.array_equal(first.view(np.uint8), outs[i][rep].cpu().numpy().view(np.uint8))
+
+
+def test_every_shape_of_the_tuned_table_under_the_automatic_pick():
+    """Each exact-shape row of csrc/tuned_table.hpp names a config by id: run the row's shape through MMBO_CONFIG_AUTO
+    against the oracle, so a row that points at a config that cannot take its shape, or computes it wrongly, is found.
+    (The two 8192^3 rows are test_cfg3_*; fp64 rows are in tests/test_dgemm_gpu.py.)"""
+    import os
+    import re
+    import gemm_mmbo_amd as G
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "gemm_mmbo_amd", "csrc", "tuned_table.hpp")).read()
+    rows = re.findall(r"^\s*\{(\d), (\d), (\d), (\d+), (\d+), (\d+), (\d+), (\w+)\((\d), (\d+)\)", text, flags=re.M)
+    assert len(rows) >= 15
+    ran = 0
+    for (dtype, ta, tb, m, n, k, batch, fam, tile, split) in rows:
+        dtype, ta, tb, m, n, k, batch, tile, split = (int(v) for v in (dtype, ta, tb, m, n, k, batch, tile, split))
+        cid = G.select_config(dtype, ta, tb, m, n, k, batch)
+        d = G.config_info(dtype, cid)
+        assert d["split_k"] == split and ("_ACC" in d["name"]) == (fam == "x16_id"), (d["name"], fam, tile, split)
+        if m * n * k >= 8192 ** 3:
+            continue
+        p = U.Problem(dtype, ta, tb, m, n, k, 1.0, 0.0, batch=batch, seed=60 + ran, dist="normal" if dtype == F16 else "uniform",
+                      c_fill="nan")
+        _run_and_check(p, -1, label=f"tuned row {dtype} {ta}{tb} {m}x{n}x{k} b{batch}")
+        ran += 1
+    assert ran >= 13
 
 
 def test_async_on_user_stream():
