@@ -18,7 +18,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libmmbo_gemm.so")
 
 EXPORTS = (
-    "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
+    "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_gemm_strided_batched_static_workspace", "mmbo_static_workspace_bytes",
+    "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
     "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_batch_xcd_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
@@ -57,6 +58,9 @@ def lib():
         L.mmbo_gemm_strided_batched.argtypes = [ci, ci, ci, sz, sz, sz, vp, vp, sz, ll, vp, sz, ll, vp, vp, sz, ll,
                                                 ci, ci, vp]
         L.mmbo_gemm_strided_batched.restype = ci
+        L.mmbo_gemm_strided_batched_static_workspace.argtypes = L.mmbo_gemm_strided_batched.argtypes
+        L.mmbo_gemm_strided_batched_static_workspace.restype = ci
+        L.mmbo_static_workspace_bytes.restype = sz
         L.mmbo_num_configs.argtypes = [ci]
         L.mmbo_num_configs.restype = ci
         L.mmbo_config_info.argtypes = [ci, ci, ctypes.POINTER(ConfigDesc)]
@@ -125,6 +129,21 @@ def gemm_strided_batched(dtype, transA, transB, m, n, k, alpha, A, lda, strideA,
     _check(lib().mmbo_gemm_strided_batched(dtype, transA, transB, m, n, k, ctypes.byref(al), _devptr(A), lda,
                                            strideA, _devptr(B), ldb, strideB, ctypes.byref(be), _devptr(C), ldc,
                                            strideC, batch, config_id, _stream_handle(stream)))
+
+
+def gemm_strided_batched_static_workspace(dtype, transA, transB, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C,
+                                          ldc, strideC, batch, config_id=CONFIG_AUTO, stream=None):
+    """The same GEMM without any device allocation: split-K partial sums go to the library's static per-device array
+    (static_workspace_bytes() of them); a call that needs more raises MmboError with status 8."""
+    al, be = _scalars(dtype, alpha, beta)
+    _check(lib().mmbo_gemm_strided_batched_static_workspace(dtype, transA, transB, m, n, k, ctypes.byref(al), _devptr(A),
+                                                            lda, strideA, _devptr(B), ldb, strideB, ctypes.byref(be),
+                                                            _devptr(C), ldc, strideC, batch, config_id,
+                                                            _stream_handle(stream)))
+
+
+def static_workspace_bytes():
+    return lib().mmbo_static_workspace_bytes()
 
 
 def num_configs(dtype):

@@ -53,13 +53,15 @@ def _units():
 
 
 def _deps():
-    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".hip", ".txt"))] + \
+    """What every translation unit depends on besides its own source: the kernel headers and the C header."""
+    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".txt"))] + \
            [os.path.join(HERE, "..", "include", "mmbo_gemm.h")]
 
 
 def _compile(unit, force, newest_dep):
     src, obj, defs = unit
     objp = os.path.join(OBJ, obj)
+    newest_dep = max(newest_dep, os.path.getmtime(os.path.join(CSRC, src)))
     if not force and os.path.exists(objp) and os.path.getmtime(objp) >= newest_dep:
         return obj, "up to date"
     cmd = [HIPCC] + FLAGS + defs + ["-c", os.path.join(CSRC, src), "-o", objp]

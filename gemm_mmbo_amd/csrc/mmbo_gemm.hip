@@ -121,6 +121,33 @@ int workspace(hipStream_t stream, size_t bytes, char **out)
     return MMBO_OK;
 }
 
+// The workspace of the entry point that allocates nothing: one array per device in the library's own image, there from
+// the moment the code object is loaded until the process ends.  In host code the array's name is only a handle: the
+// device address of each GPU's copy comes from hipGetSymbolAddress, once per device, and that pointer is what the
+// kernels get.  Nothing in it has to start at zero: every partial sum a GEMM reads was written by that same GEMM.
+constexpr size_t kScratchPartialBytes = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchPartialBytes];
+std::mutex g_scratch_mutex;
+char *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(char **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e);
+        if (!p) return MMBO_ERR_WORKSPACE;
+        g_scratch_ptr[dev] = static_cast<char *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return MMBO_OK;
+}
+
 // ---- table ------------------------------------------------------------------------------------
 template <int DTYPE, int TILE>
 hipError_t dispatch_tile(int tile, int ta, int tb, const GemmArgs &a, hipStream_t s)
@@ -524,14 +551,19 @@ int mmbo_release_workspace(void)
     return MMBO_OK;
 }
 
+size_t mmbo_static_workspace_bytes(void) { return kScratchPartialBytes; }
+
 }  // extern "C"
 
 namespace {
 
+// Where the partial sums of a split-K config go.
+enum class WsSource { kLibrary, kStatic };
+
 int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
               const void *alpha, const void *A, size_t lda, long long strideA,
               const void *B, size_t ldb, long long strideB, const void *beta, void *C,
-              size_t ldc, long long strideC, int batch, int config_id, void *stream)
+              size_t ldc, long long strideC, int batch, int config_id, void *stream, WsSource ws_source)
 {
     if (!valid_dtype(dtype)) return MMBO_ERR_INVALID_DTYPE;
     if ((transA & ~1) || (transB & ~1)) return MMBO_ERR_INVALID_OP;
@@ -635,16 +667,22 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
-    // Split-K: the partial sums go to the stream's own workspace, and both launches that use it (the
+    // Split-K: the partial sums go to the stream's own workspace (or the static one), and both launches that use it (the
     // GEMM and the reduction, which adds the splits in ascending order) are queued before the lock on the workspace
     // table is given up.
     std::unique_lock<std::mutex> ws_lock;
     if (split > 1) {
         const size_t bytes = (size_t)split * batch * m * n * sizeof(float);
         char *base = nullptr;
-        ws_lock = std::unique_lock<std::mutex>(g_ws_mutex);
-        int rc = workspace(s, bytes, &base);
-        if (rc != MMBO_OK) return rc;
+        if (ws_source == WsSource::kStatic) {
+            if (bytes > kScratchPartialBytes) return MMBO_ERR_WORKSPACE;
+            int rc = static_scratch(&base);
+            if (rc != MMBO_OK) return rc;
+        } else {
+            ws_lock = std::unique_lock<std::mutex>(g_ws_mutex);
+            int rc = workspace(s, bytes, &base);
+            if (rc != MMBO_OK) return rc;
+        }
         a.ws = reinterpret_cast<float *>(base);
     }
     hipError_t e;
@@ -673,7 +711,16 @@ int mmbo_gemm_strided_batched(int dtype, int transA, int transB, size_t m, size_
                               size_t ldc, long long strideC, int batch, int config_id, void *stream)
 {
     return gemm_impl(dtype, transA, transB, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch,
-                     config_id, stream);
+                     config_id, stream, WsSource::kLibrary);
+}
+
+int mmbo_gemm_strided_batched_static_workspace(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+                                               const void *alpha, const void *A, size_t lda, long long strideA,
+                                               const void *B, size_t ldb, long long strideB, const void *beta, void *C,
+                                               size_t ldc, long long strideC, int batch, int config_id, void *stream)
+{
+    return gemm_impl(dtype, transA, transB, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch,
+                     config_id, stream, WsSource::kStatic);
 }
 
 int mmbo_gemm(int dtype, int transA, int transB, size_t m, size_t n, size_t k, const void *alpha,

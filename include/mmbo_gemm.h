@@ -63,7 +63,8 @@ typedef enum mmbo_status {
     MMBO_ERR_INVALID_CONFIG = 5,    /* config_id outside the table, or not usable for this call */
     MMBO_ERR_HIP = 6,               /* a HIP runtime call failed; mmbo_last_hip_error() has the code */
     MMBO_ERR_NO_DEVICE = 7,         /* no gfx950 device is current */
-    MMBO_ERR_WORKSPACE = 8          /* split-K workspace could not be allocated */
+    MMBO_ERR_WORKSPACE = 8          /* split-K workspace could not be allocated, or the partial sums of this call do
+                                       not fit the static workspace of the entry point that allocates nothing */
 } mmbo_status;
 
 /* One row of the tile-config table (reference: the {MT0I, MT1J, threads} triples of
@@ -130,6 +131,25 @@ int mmbo_chip_block_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsi
  * same panel of A or B share an L2.  The reference has no batches in its launcher (src/gemm/driver.h:49-59) and one
  * L2.  A bijection of [0, tiles*batch); needs batch % 8 == 0.  Pure host logic. */
 int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, unsigned *tile, unsigned *batch_index);
+
+/* The same GEMM for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose launcher allocates nothing either, but
+ * has no split-K: GlobalSplitU 1, src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:69).  Arguments, results and status codes
+ * are those of mmbo_gemm_strided_batched (batch = 1 with zero strides is mmbo_gemm); the results are the same bit for bit.
+ * The difference: the partial sums of a config with GlobalSplitU > 1 live in an array that is part
+ * of the library's device image (mmbo_static_workspace_bytes() bytes of partial sums, 32 MiB, held by every GPU the
+ * library runs on until the process ends) instead of in memory from hipMalloc, and the call makes no hipMalloc, hipFree
+ * or other allocating call.  A call whose partial sums (GlobalSplitU x batch x m x n x 4 bytes; mmbo_config_info of
+ * mmbo_select_config's pick gives GlobalSplitU) do not fit is refused with MMBO_ERR_WORKSPACE and launches nothing;
+ * configs without split-K need no workspace and always run.  All calls on one GPU share that GPU's array: two such
+ * split-K calls that overlap in time on one GPU (different streams, or different host threads) race on it -- keep them
+ * on one stream.  The first call on a device looks the array's address up (hipGetSymbolAddress), once. */
+int mmbo_gemm_strided_batched_static_workspace(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
+                                               const void *alpha, const void *A, size_t lda, long long strideA,
+                                               const void *B, size_t ldb, long long strideB,
+                                               const void *beta, void *C, size_t ldc, long long strideC,
+                                               int batch, int config_id, void *stream);
+size_t mmbo_static_workspace_bytes(void);
 
 /* Release the split-K workspaces held for the current device (one per stream that ran a split-K config; allocated
  * lazily, grown on demand, reused across calls).  Waits for the device.  The reference never frees what it loads
