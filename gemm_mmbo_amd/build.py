@@ -52,16 +52,23 @@ def _units():
     return units
 
 
-def _deps():
-    """What every translation unit depends on besides its own source: the kernel headers and the C header."""
-    return [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".txt"))] + \
-           [os.path.join(HERE, "..", "include", "mmbo_gemm.h")]
+def _deps(src, seen=None):
+    """The files a source depends on: itself and, recursively, everything it includes with #include "..."."""
+    import re
+    seen = seen if seen is not None else set()
+    path = os.path.normpath(src)
+    if path in seen or not os.path.exists(path):
+        return seen
+    seen.add(path)
+    for inc in re.findall(r'^\s*#\s*include\s+"([^"]+)"', open(path).read(), flags=re.M):
+        _deps(os.path.join(os.path.dirname(path), inc), seen)
+    return seen
 
 
 def _compile(unit, force, newest_dep):
     src, obj, defs = unit
     objp = os.path.join(OBJ, obj)
-    newest_dep = max(newest_dep, os.path.getmtime(os.path.join(CSRC, src)))
+    newest_dep = max([newest_dep] + [os.path.getmtime(p) for p in _deps(os.path.join(CSRC, src))])
     if not force and os.path.exists(objp) and os.path.getmtime(objp) >= newest_dep:
         return obj, "up to date"
     cmd = [HIPCC] + FLAGS + defs + ["-c", os.path.join(CSRC, src), "-o", objp]
@@ -73,7 +80,8 @@ def _compile(unit, force, newest_dep):
 
 def build(force=False, verbose=True, jobs=None):
     os.makedirs(OBJ, exist_ok=True)
-    newest = max(os.path.getmtime(p) for p in _deps())
+    extra = os.path.join(CSRC, "extra_units.txt")
+    newest = max(os.path.getmtime(p) for p in (os.path.abspath(__file__), extra) if os.path.exists(p))
     units = _units()
     jobs = jobs or min(8, os.cpu_count() or 1)
     with ThreadPoolExecutor(max_workers=jobs) as ex:

@@ -179,11 +179,7 @@ struct SliceFrags {
 
 }  // namespace ring
 
-// ABLATE is a timing probe in the spirit of the reference's error_kernel_000.s / test_main_loop.s (kernels
-// with parts removed to find the ceiling of what is left; results are wrong by design): bit 0 drops the
-// global->LDS loads, bit 1 the LDS fragment reads, bit 2 the MFMAs, bit 3 writes the main loop's clock64 and
-// wall_clock64 spans to args.ws.  The library only instantiates ABLATE = 0.
-template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
 struct RingCfg {
     static constexpr int NW = WM * WN, NT = NW * 64;
     static constexpr int BK = ring::Slice<T>::BK;
@@ -201,12 +197,12 @@ struct RingCfg {
     static constexpr int NMFMA = 2 * FM * FN * MPK;
 };
 
-template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0>
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_ring_kernel(const GemmArgs args)
 {
     using namespace ring;
-    using Cfg = RingCfg<T, TA, TB, BM, BN, WM, WN, DEPTH, ABLATE>;
+    using Cfg = RingCfg<T, TA, TB, BM, BN, WM, WN, DEPTH>;
     using TileA = typename Cfg::TileA;
     using TileB = typename Cfg::TileB;
     using FragA = typename Cfg::FragA;
@@ -247,7 +243,6 @@ gemm_ring_kernel(const GemmArgs args)
 
     // slice s goes to ring buffer s % DEPTH; `buf` is that index, kept by the caller
     auto issue_slice = [&](int s, int buf) {
-        if constexpr (ABLATE & 1) return;
         char *dst = lds + buf * Cfg::SLICE_BYTES;
         const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
 #pragma unroll
@@ -264,19 +259,6 @@ gemm_ring_kernel(const GemmArgs args)
     const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
     FragA fa[2];
     FragB fb[2];
-    if constexpr (ABLATE != 0) {      // keep the probes' registers defined
-        const uint32_t va = (ESZ == 2 ? 0x3c003c00u : 0x3f800000u) + (uint32_t)lane;
-#pragma unroll
-        for (int q = 0; q < 2; ++q)
-#pragma unroll
-            for (int kg = 0; kg < 2; ++kg) {
-#pragma unroll
-                for (int f = 0; f < FM; ++f) fa[q].x[kg][f] = u32x4{va, va, va, va};
-#pragma unroll
-                for (int f = 0; f < FN; ++f) fb[q].x[kg][f] = u32x4{va, va, va, va};
-            }
-    }
-
     f32x16 acc[FM][FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -287,7 +269,6 @@ gemm_ring_kernel(const GemmArgs args)
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
-        if constexpr (ABLATE & 2) return;
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
         b.read_all(t + TileA::BYTES, adB);
@@ -312,19 +293,18 @@ gemm_ring_kernel(const GemmArgs args)
             constexpr int m = decltype(M)::value;
             // consecutive MFMAs go to different accumulators
             constexpr int kg = m / (FM * FN * MPK), tt = (m / (FM * FN)) % MPK, i = (m / FN) % FM, j = m % FN;
-            if constexpr (!(ABLATE & 4)) {
-                if constexpr (ESZ == 2)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ca.x[kg][i]),
-                                                                       __builtin_bit_cast(f16x8, cb.x[kg][j]), acc[i][j], 0, 0, 0);
-                else {
-                    // (through locals: bit-casting a vector-element expression directly picked element 0)
-                    const uint32_t ua = ca.x[kg][i][tt], ub = cb.x[kg][j][tt];
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, ua),
-                                                                     __builtin_bit_cast(float, ub), acc[i][j], 0, 0, 0);
-                }
+            if constexpr (ESZ == 2)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ca.x[kg][i]),
+                                                                   __builtin_bit_cast(f16x8, cb.x[kg][j]), acc[i][j], 0, 0, 0);
+            else {
+                // (through locals: bit-casting a vector-element expression directly picked element 0)
+                const uint32_t ua = ca.x[kg][i][tt], ub = cb.x[kg][j][tt];
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, ua),
+                                                                 __builtin_bit_cast(float, ub), acc[i][j], 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (!(ABLATE & 2) && m < READ_SPAN) {
+            // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
+            // pad the gap with an s_nop, which costs an issue slot like any other instruction)
+            if constexpr (m < READ_SPAN) {
                 constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
                 static_for<r1 - r0>([&](auto RR) {
                     constexpr int r = r0 + decltype(RR)::value;
@@ -332,7 +312,7 @@ gemm_ring_kernel(const GemmArgs args)
                     else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
-            if constexpr (!(ABLATE & 1)) {
+            {
                 // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
                 constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
                 static_for<l1 - l0>([&](auto LL) {
@@ -362,9 +342,6 @@ gemm_ring_kernel(const GemmArgs args)
     } while (0)
 #define MMBO_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
 #define MMBO_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
-
-    long long t_clk = 0, t_wall = 0;
-    if constexpr (ABLATE & 8) { t_clk = clock64(); t_wall = wall_clock64(); }
 
     // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
     // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free; this
@@ -413,12 +390,6 @@ gemm_ring_kernel(const GemmArgs args)
     for (; s < n_slice; s += 2) {
         step(s, fa[0], fb[0], fa[1], fb[1]);
         if (s + 1 < n_slice) step(s + 1, fa[1], fb[1], fa[0], fb[0]);
-    }
-    if constexpr (ABLATE & 8) {
-        if (tid == 0 && blockIdx.x == args.nwg0 * args.nwg1 / 3) {
-            reinterpret_cast<long long *>(args.ws)[0] = clock64() - t_clk;
-            reinterpret_cast<long long *>(args.ws)[1] = wall_clock64() - t_wall;
-        }
     }
 #undef MMBO_BARRIER
 #undef MMBO_WAIT_VM

@@ -47,35 +47,45 @@ using ring::static_for;
     "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239" , \
     "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
 
-// acc block BASE/4 += A-fragment x B-fragment.  NACC = accumulator registers the kernel owns (64, 128 or 256).
+// The 64 accumulator blocks a[4q : 4q+3], spelled out: an asm statement names its registers and its clobbers as literals.
+#define MMBO_ACC_BLOCKS(X) \
+    X(0,1,2,3) X(4,5,6,7) X(8,9,10,11) X(12,13,14,15) X(16,17,18,19) X(20,21,22,23) X(24,25,26,27) X(28,29,30,31) \
+    X(32,33,34,35) X(36,37,38,39) X(40,41,42,43) X(44,45,46,47) X(48,49,50,51) X(52,53,54,55) X(56,57,58,59) X(60,61,62,63) \
+    X(64,65,66,67) X(68,69,70,71) X(72,73,74,75) X(76,77,78,79) X(80,81,82,83) X(84,85,86,87) X(88,89,90,91) X(92,93,94,95) \
+    X(96,97,98,99) X(100,101,102,103) X(104,105,106,107) X(108,109,110,111) X(112,113,114,115) X(116,117,118,119) X(120,121,122,123) X(124,125,126,127) \
+    X(128,129,130,131) X(132,133,134,135) X(136,137,138,139) X(140,141,142,143) X(144,145,146,147) X(148,149,150,151) X(152,153,154,155) X(156,157,158,159) \
+    X(160,161,162,163) X(164,165,166,167) X(168,169,170,171) X(172,173,174,175) X(176,177,178,179) X(180,181,182,183) X(184,185,186,187) X(188,189,190,191) \
+    X(192,193,194,195) X(196,197,198,199) X(200,201,202,203) X(204,205,206,207) X(208,209,210,211) X(212,213,214,215) X(216,217,218,219) X(220,221,222,223) \
+    X(224,225,226,227) X(228,229,230,231) X(232,233,234,235) X(236,237,238,239) X(240,241,242,243) X(244,245,246,247) X(248,249,250,251) X(252,253,254,255)
+
+// acc block BASE/4 += A-fragment x B-fragment.  The statement clobbers exactly the four registers it writes.  (With every
+// accumulation register in every MFMA's clobber list the compiler pads each pair of neighbouring asm statements with an
+// s_nop: for statements it cannot look into, it assumes a result-forwarding hazard whenever what one writes overlaps what
+// the next names.  An s_nop is an issue slot like any other instruction, and there was one for almost every MFMA.)
+// Nothing else may ever hold a value in these registers: acc_zero claims all of them for the kernel, and
+// tests/test_kernel_asm.py checks that no compiler-generated instruction of these kernels names an accumulation register.
 template <int BASE, int NACC>
 __device__ __forceinline__ void mfma_acc(const u32x4 &a, const u32x4 &b)
 {
     static_assert(BASE % 4 == 0 && BASE + 4 <= NACC, "accumulator block out of range");
-    if constexpr (NACC > 128)
-        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
-    else if constexpr (NACC > 64)
-        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
-    else
-        asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63);
+#define X(r0, r1, r2, r3)                                                                                     \
+    if constexpr (BASE == r0)                                                                                 \
+        asm volatile("v_mfma_f32_16x16x32_f16 a[" #r0 ":" #r3 "], %0, %1, a[" #r0 ":" #r3 "]" ::"v"(a), "v"(b) \
+                     : "a" #r0, "a" #r1, "a" #r2, "a" #r3);
+    MMBO_ACC_BLOCKS(X)
+#undef X
 }
 // fp32: acc block BASE/4 += (one k of four per lane group) A x B; called four times per fragment pair
 template <int BASE, int NACC>
 __device__ __forceinline__ void mfma_acc_f32(uint32_t a, uint32_t b)
 {
     static_assert(BASE % 4 == 0 && BASE + 4 <= NACC, "accumulator block out of range");
-    if constexpr (NACC > 128)
-        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
-    else if constexpr (NACC > 64)
-        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
-    else
-        asm volatile("v_mfma_f32_16x16x4_f32 a[%2:%3], %0, %1, a[%2:%3]"
-                     :: "v"(a), "v"(b), "n"(BASE), "n"(BASE + 3) : MMBO_AGPR_0_63);
+#define X(r0, r1, r2, r3)                                                                                    \
+    if constexpr (BASE == r0)                                                                                \
+        asm volatile("v_mfma_f32_16x16x4_f32 a[" #r0 ":" #r3 "], %0, %1, a[" #r0 ":" #r3 "]" ::"v"(a), "v"(b) \
+                     : "a" #r0, "a" #r1, "a" #r2, "a" #r3);
+    MMBO_ACC_BLOCKS(X)
+#undef X
 }
 template <int NACC>
 __device__ __forceinline__ void acc_zero()
@@ -282,14 +292,11 @@ struct X16Cfg {
     static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
 };
 
-// ABLATE: timing probe as in gemm_ring.hpp (bit 0 no direct loads, bit 1 no LDS reads, bit 2 no MFMAs: results are
-// wrong by design; bit 3 writes each work-group's start, loop start, loop end and end times (100 MHz counter) to
-// args.ws[4 * work-group ..]).  The library only instantiates ABLATE = 0.
 // PAIR: fetch two slices of one operand per iteration (see mfma_and_read); on when an operand is k-contiguous.
 // EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
 // one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
-template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, int ABLATE = 0, bool PAIR = (TA || !TB),
+template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, bool PAIR = (TA || !TB),
           int EVEN_OP = (TA ? 0 : 1)>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_x16_kernel(const GemmArgs args)
@@ -309,8 +316,6 @@ gemm_x16_kernel(const GemmArgs args)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WM, wn = wave / WM;
-    long long t_probe[4] = {0, 0, 0, 0};
-    if constexpr ((ABLATE & 8) != 0) t_probe[0] = wall_clock64();
 
     // A work-group walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...: the host launches one work-group per tile,
     // or, for the 256 x 256 tiles on grids larger than the chip, one per CU (persistent).  Staying resident saves the
@@ -367,7 +372,6 @@ gemm_x16_kernel(const GemmArgs args)
                                              MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024), 16, 0, 0);
     };
     auto issue_slice = [&](int s, int buf) {
-        if constexpr (ABLATE & 1) return;
         char *dst = lds + buf * Cfg::SLICE_BYTES;
         const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
         static_for<BATCH>([&](auto L) { issue_load(L, pa, pb, dst); });
@@ -389,22 +393,10 @@ gemm_x16_kernel(const GemmArgs args)
     const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
     FragA fa[2];
     FragB fb[2];
-    if constexpr (ABLATE != 0) {      // the probes' MFMAs must see operand bits like the real ones: power depends on them
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(args.A);
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-#pragma unroll
-            for (int f = 0; f < FM; ++f) fa[q].x[f] = src[(q * 16 + f) * 64 + lane];
-#pragma unroll
-            for (int f = 0; f < FN; ++f) fb[q].x[f] = src[(q * 16 + 8 + f) * 64 + lane];
-        }
-    }
-
     acc_zero<NACC>();
 
     const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
-        if constexpr (ABLATE & 2) return;
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
         b.read_all(t + TileA::BYTES, adB);
@@ -439,12 +431,11 @@ gemm_x16_kernel(const GemmArgs args)
             // fp32 walks the blocks four times, once per k register, so an accumulator recurs every FM*FN MFMAs
             constexpr int tt = m / (FM * FN), ij = m % (FM * FN);
             constexpr int i = ij / FN, j = (i & 1) ? FN - 1 - ij % FN : ij % FN;
-            if constexpr (!(ABLATE & 4)) {
-                if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
-                else mfma_acc_f32<(i * FN + j) * 4, NACC>(ca.x[i][tt], cb.x[j][tt]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (!(ABLATE & 2) && m < READ_SPAN) {
+            if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
+            else mfma_acc_f32<(i * FN + j) * 4, NACC>(ca.x[i][tt], cb.x[j][tt]);
+            // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
+            // pad the gap with an s_nop, which costs an issue slot like any other instruction)
+            if constexpr (m < READ_SPAN) {
                 constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
                 static_for<r1 - r0>([&](auto RR) {
                     constexpr int r = r0 + decltype(RR)::value;
@@ -452,7 +443,7 @@ gemm_x16_kernel(const GemmArgs args)
                     else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
-            if constexpr (!(ABLATE & 1) && load_mode != 0 && PAIR) {
+            if constexpr (load_mode != 0 && PAIR) {
                 constexpr int l0 = (2 * LOP * m + NMFMA) / (2 * NMFMA), l1 = (2 * LOP * (m + 1) + NMFMA) / (2 * NMFMA);
                 static_for<l1 - l0>([&](auto LL) {
                     constexpr int l = l0 + decltype(LL)::value;
@@ -462,7 +453,7 @@ gemm_x16_kernel(const GemmArgs args)
                     }
                 });
             }
-            if constexpr (!(ABLATE & 1) && load_mode != 0 && !PAIR) {
+            if constexpr (load_mode != 0 && !PAIR) {
                 // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
                 constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
                 static_for<l1 - l0>([&](auto LL) {
@@ -484,17 +475,6 @@ gemm_x16_kernel(const GemmArgs args)
 #define MMBO_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
 #define MMBO_WAIT_LGKM0() asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory")
 
-    // Without the MFMAs nothing reads the fragments, and a register whose asynchronous LDS read is still in flight
-    // could be handed to something else (a load address, say) before the data lands in it: keep them live past the wait.
-    auto keep_alive = [&](const FragA &a, const FragB &b) {
-        if constexpr ((ABLATE & 4) != 0) {
-#pragma unroll
-            for (int f = 0; f < FM; ++f) asm volatile("" :: "v"(a.x[f]));
-#pragma unroll
-            for (int f = 0; f < FN; ++f) asm volatile("" :: "v"(b.x[f]));
-        }
-    };
-
     // Invariant at the top of iteration s (after barrier B_s): register set s&1 holds slice s; slice s+1 is
     // resident in LDS; every wavefront has finished reading slices <= s, so buffer s % DEPTH is free (and, for the
     // operand whose turn it is in paired mode, buffer (s-1) % DEPTH too); the loads of the later slices are in flight.
@@ -503,7 +483,6 @@ gemm_x16_kernel(const GemmArgs args)
     // that may stay in flight.
     int buf = 0;                                                     // s % DEPTH
     int s = 0;
-    if constexpr ((ABLATE & 8) != 0) t_probe[1] = wall_clock64();
     if constexpr (!PAIR) {
 #pragma unroll
         for (int q = 0; q < DEPTH; ++q)
@@ -512,7 +491,6 @@ gemm_x16_kernel(const GemmArgs args)
         MMBO_BARRIER();                                                  // slice 0 resident
         read_slice(fa[0], fb[0], 0);
         MMBO_WAIT_LGKM0();
-        keep_alive(fa[0], fb[0]);
         if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
 
@@ -521,7 +499,6 @@ gemm_x16_kernel(const GemmArgs args)
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
             MMBO_WAIT_LGKM0();
-            keep_alive(na, nb);
             MMBO_WAIT_VM(BATCH * (DEPTH - 2));
             MMBO_BARRIER();
             buf = nbuf;
@@ -533,7 +510,6 @@ gemm_x16_kernel(const GemmArgs args)
             const bool load = s + DEPTH < n_slice;
             mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, s + DEPTH, buf);
             MMBO_WAIT_LGKM0();
-            keep_alive(na, nb);
             if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
             MMBO_BARRIER();
             buf = nbuf;
@@ -553,13 +529,11 @@ gemm_x16_kernel(const GemmArgs args)
         constexpr std::integral_constant<int, EVEN_OP> OPX{};
         constexpr std::integral_constant<int, 1 - EVEN_OP> OPY{};
         // prologue: X slices 0 .. DEPTH-2, Y slices 0 .. DEPTH-1, slice by slice (iteration 0 brings X's DEPTH-1 and DEPTH)
-        if constexpr (!(ABLATE & 1)) {
 #pragma unroll
-            for (int q = 0; q < DEPTH; ++q) {
-                if (q < n_slice) {
-                    if (q < DEPTH - 1) static_for<LA>([&](auto I) { issue_op_load(OPX, I, q, q); });
-                    static_for<LB>([&](auto I) { issue_op_load(OPY, I, q, q); });
-                }
+        for (int q = 0; q < DEPTH; ++q) {
+            if (q < n_slice) {
+                if (q < DEPTH - 1) static_for<LA>([&](auto I) { issue_op_load(OPX, I, q, q); });
+                static_for<LB>([&](auto I) { issue_op_load(OPY, I, q, q); });
             }
         }
         constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
@@ -567,7 +541,6 @@ gemm_x16_kernel(const GemmArgs args)
         MMBO_BARRIER();                                                  // slice 0 resident
         read_slice(fa[0], fb[0], 0);
         MMBO_WAIT_LGKM0();
-        keep_alive(fa[0], fb[0]);
         if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - 2 * BATCH); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
 
@@ -580,7 +553,6 @@ gemm_x16_kernel(const GemmArgs args)
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
             MMBO_WAIT_LGKM0();
-            keep_alive(na, nb);
             MMBO_WAIT_VM(KEEP);
             MMBO_BARRIER();
             buf = nbuf;
@@ -596,7 +568,6 @@ gemm_x16_kernel(const GemmArgs args)
             const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
             mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, s + DEPTH, buf);
             MMBO_WAIT_LGKM0();
-            keep_alive(na, nb);
             const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP;
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
             constexpr int KMAX = 2 * (LA > LB ? LA : LB) * 3;
@@ -648,7 +619,6 @@ gemm_x16_kernel(const GemmArgs args)
         });
         __syncthreads();            // the next tile's direct loads overwrite buffer 0
     }
-    if constexpr ((ABLATE & 8) != 0) t_probe[2] = wall_clock64();
     // the last MFMAs' results must have landed before they are read back
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
@@ -813,15 +783,6 @@ gemm_x16_kernel(const GemmArgs args)
                 p[r] = (T)o;
             }
         });
-    }
-    if constexpr ((ABLATE & 8) != 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        t_probe[3] = wall_clock64();
-        if (tid == 0) {
-            long long *o = reinterpret_cast<long long *>(args.ws) + 4 * (size_t)tile;
-            o[0] = t_probe[0]; o[1] = t_probe[1]; o[2] = t_probe[2]; o[3] = t_probe[3];
-        }
-        t_probe[0] = t_probe[3];
     }
     }   // tiles of this work-group
 }

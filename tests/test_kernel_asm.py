@@ -210,9 +210,14 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
                     used.update(range(int(a, 0), int(b, 0) + 1))
                 used.update(int(a, 0) for a in re.findall(r"\ba\[(\w+)\]", t))
                 # no accumulation register may appear outside the MFMAs, the zeroing and the read-back
+                # (an MFMA statement only declares the four registers it writes as clobbered, so the compiler believes the
+                # others free at that point: it must never have put a value of its own into one -- the only writes are
+                # the MFMAs and the zeroing at the start of a tile)
                 if re.search(r"\ba\[?\d", t):
                     assert t.startswith(("v_mfma_f32_16x16x32_f16", "v_mfma_f32_16x16x4_f32", "v_accvgpr_write_b32",
                                          "v_accvgpr_read_b32")), (name, t)
+                    if t.startswith("v_accvgpr_write_b32"):
+                        assert re.match(r"v_accvgpr_write_b32 a\[?\w+\]?, 0$", t), (name, t)
             m = re.search(r"\.amdhsa_kernel " + re.escape(name) + r"\b.*?\.amdhsa_next_free_vgpr (\d+).*?\.amdhsa_accum_offset (\d+)",
                           text, re.S)
             assert m, name
