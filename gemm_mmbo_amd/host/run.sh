@@ -3,9 +3,16 @@
 # N=2048, K=384, ldc=44160 > M), plus the five benchmark configurations of this library.
 #   ./run.sh hpl [dtype]      the reference's HPL trailing-update sweep, best config per size (type 1)
 #   ./run.sh configs          the five benchmark configurations with the table's pick (type 0)
+#   ./run.sh report MODE [args]   machine-readable records (JSON lines on stdout, --json/--csv FILE) with roofline
+#                                 fractions, an fp64 check and the rocprofv3 commands per shape: MODE = configs | hpl |
+#                                 shapes SPEC...  (python -m gemm_mmbo_amd.report)
 cd "$(dirname "$0")"
 mode=${1:-configs}
-if [ "$mode" = hpl ]; then
+if [ "$mode" = report ]; then
+  shift
+  cd ../.. && python3 -m gemm_mmbo_amd.report "$@"
+  exit $?
+elif [ "$mode" = hpl ]; then
   dt=${2:-d}
   for M in {44160..384..-3840}; do
     ./benchmark 1 ${M} 2048 384 ${M} 2048 44160 N T ${dt} 1 -1 1 || exit 1

@@ -566,6 +566,44 @@ def test_cpp_benchmark_main_modes():
     assert r.returncode == 2
 
 
+def test_report_driver_writes_parsable_records(tmp_path):
+    """python -m gemm_mmbo_amd.report (the sweep driver behind host/run.sh report; reference: src/gemm/run.sh:1-5 over
+    src/gemm/benchmark.cc:89-109): two small shapes, JSON lines on stdout and in a file, a CSV with the same rows, the
+    roofline arithmetic, the fp64 cross-check and the profiling commands."""
+    import csv
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    jpath, cpath = str(tmp_path / "r.jsonl"), str(tmp_path / "r.csv")
+    r = subprocess.run([sys.executable, "-m", "gemm_mmbo_amd.report", "shapes", "h,T,N,512,384,1024,2,1,0.5", "s,N,N,257,131,1000",
+                        "--json", jpath, "--csv", cpath, "--reps", "5", "--print-profile-commands"],
+                       cwd=root, capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stderr[-2000:]
+    recs = [json.loads(l) for l in r.stdout.splitlines() if l.startswith("{")]
+    assert recs == [json.loads(l) for l in open(jpath)]
+    rows = list(csv.DictReader(open(cpath)))
+    assert len(recs) == 2 and len(rows) == 2
+    h, s = recs
+    assert (h["dtype"], h["transA"], h["transB"], h["m"], h["n"], h["k"], h["batch"], h["beta"]) == ("h", "T", "N", 512, 384, 1024, 2, 0.5)
+    assert h["algorithmic_bytes"] == 2 * (512 * 1024 + 1024 * 384 + 2 * 512 * 384) * 2          # beta != 0: C counted twice
+    assert s["algorithmic_bytes"] == (257 * 1000 + 1000 * 131 + 257 * 131) * 4
+    for rec, row, limit in ((h, rows[0], 2e-2), (s, rows[1], 1e-5 * 1000 ** 0.5)):
+        assert 0 < rec["gpu_ms_min"] <= rec["gpu_ms_median"] <= rec["gpu_ms_max"]
+        flops = 2.0 * rec["m"] * rec["n"] * rec["k"] * rec["batch"]
+        assert abs(rec["tflops"] - flops / rec["gpu_ms_median"] * 1e-9) <= 0.02 * rec["tflops"] + 0.01
+        assert rec["bound"] in ("mfma", "hbm") and 0 < rec["frac_of_bound"] <= 1.0 and 0 < rec["frac_of_peak"] <= 1.0
+        assert rec["frac_of_bound"] >= rec["frac_of_peak"]
+        assert rec["max_rel_err"] <= limit and "fp64" in rec["checked_against"]
+        assert rec["config"] and row["config"] == rec["config"] and float(row["gpu_ms_median"]) == rec["gpu_ms_median"]
+    cmds = [l for l in r.stdout.splitlines() if l.startswith("# ")]
+    assert len(cmds) == 8 and all("rocprofv3" in c and " -- python3 -m gemm_mmbo_amd.report shapes " in c for c in cmds)
+    assert sum("--kernel-trace --stats" in c for c in cmds) == 2 and sum("FETCH_SIZE" in c for c in cmds) == 2
+    bad = subprocess.run([sys.executable, "-m", "gemm_mmbo_amd.report", "shapes", "q,N,N,1,1,1"], cwd=root, capture_output=True, text=True)
+    assert bad.returncode != 0
+
+
 def test_mfma_ceiling_probe_reports_plausible_numbers():
     """mmbo_probe_mfma_ceiling: a register-only MFMA loop cannot beat the published peaks, and constant operands
     are never slower than random ones (the chip clocks down under power)."""
