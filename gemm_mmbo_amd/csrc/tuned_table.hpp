@@ -36,11 +36,11 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 128, 4096, 8192, 1, ring_id(3, 8), 108.8f},
     {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 423.9f},
     {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 442.8f},
-    {0, 0, 0, 2048, 2048, 2048, 1, ring_id(3, 1), 117.5f},
+    {0, 0, 0, 2048, 2048, 2048, 1, ring_id(2, 1), 128.6f},
     {1, 0, 0, 2048, 2048, 2048, 1, x16_id(2, 1), 761.2f},
     {0, 0, 1, 44160, 2048, 384, 1, x16_id(2, 1), 120.5f},
-    {0, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 145.3f},
-    {1, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 1330.0f},
+    {0, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 146.1f},
+    {1, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 1355.2f},
     {0, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 143.6f},
     {1, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 1245.0f},
     {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // fp64 ids are rows of kTilesF64; the reference's HPL trailing update (src/gemm/run.sh:2-5)

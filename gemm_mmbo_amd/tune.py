@@ -11,6 +11,7 @@ GPU it runs on:
     python -m gemm_mmbo_amd.tune shapes.txt --dump t.json    # also write every config's time per shape
 
 For every shape it prints the ranking and one line in the table's syntax; paste the lines into kTuned[] and rebuild.
+The fastest config only enters a line after its result has passed a check against the library's fp64 kernel.
 Configs that do not apply to a shape (the ring kernels on ragged shapes or on operands that are not 16-byte aligned: the
 operands here are tightly packed) are skipped, as the C ABI refuses them.
 """
@@ -50,13 +51,41 @@ def time_config(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, cfg, reps)
     except G.MmboError:
         return None
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(reps):
-        run()
-    e1.record(stream)
+    # median over five groups of `reps` back-to-back launches
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+    ev[0].record(stream)
+    for g in range(5):
+        for _ in range(reps):
+            run()
+        ev[g + 1].record(stream)
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / reps
+    return sorted(ev[g].elapsed_time(ev[g + 1]) / reps for g in range(5))[2]
+
+
+def table_id(G, dtype, cfg):
+    """A config id in the syntax of csrc/tuned_table.hpp: ring_id(tile, GlobalSplitU) / x16_id(tile, GlobalSplitU) for the
+    direct-to-LDS families (tile = row of kRingTiles / kX16Tiles), the plain number otherwise (staged ids, fp64 rows)."""
+    if dtype == G.F64:
+        return str(cfg)
+    d = G.config_info(dtype, cfg)
+    if "DTL1" not in d["name"]:
+        return str(cfg)
+    fam = [c for c in range(G.num_configs(dtype))
+           if ("DTL1" in G.config_info(dtype, c)["name"]) and (("_ACC" in G.config_info(dtype, c)["name"]) == ("_ACC" in d["name"]))
+           and G.config_info(dtype, c)["split_k"] == 1]
+    ntiles = len(fam)
+    tile = (cfg - fam[0]) % ntiles
+    return f"{'x16_id' if '_ACC' in d['name'] else 'ring_id'}({tile}, {d['split_k']})"
+
+
+def passes_check(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, cfg):
+    """The candidate's result against this library's fp64 kernel on the same operands (gemm_mmbo_amd.report), within the
+    library's tolerances: a config that is fast and wrong must never enter the table."""
+    from . import report
+    d = {G.F32: "s", G.F16: "h", G.F64: "d"}[dtype]
+    rec = report.run_shape(G, torch, (d, "NT"[ta], "NT"[tb], m, n, k, batch, alpha, beta, None), 1, 1, cfg, True)
+    limit = {G.F32: 1e-5 * max(k, 1) ** 0.5, G.F16: 2e-2, G.F64: 2e-15 * max(k, 1) ** 0.5}[dtype]
+    return rec["max_rel_err"] is None or rec["max_rel_err"] <= limit
 
 
 def tune(shapes, out=sys.stdout, dump=None):
@@ -81,8 +110,11 @@ def tune(shapes, out=sys.stdout, dump=None):
         res.sort()
         pick = G.select_config(dtype, ta, tb, m, n, k, batch)
         t_pick = next((t for t, c in res if c == pick), None)
+        while res and not passes_check(G, torch, dtype, ta, tb, m, n, k, batch, alpha, beta, res[0][1]):
+            print(f"# config {res[0][1]} FAILS the result check on this shape: left out", file=out)
+            res.pop(0)
         best_t, best = res[0]
-        row = f"    {{{dtype}, {ta}, {tb}, {m}, {n}, {k}, {batch}, {best}, {flops / best_t * 1e-9:.1f}f}},"
+        row = f"    {{{dtype}, {ta}, {tb}, {m}, {n}, {k}, {batch}, {table_id(G, dtype, best)}, {flops / best_t * 1e-9:.1f}f}},"
         rows.append(row)
         print(f"# dtype {dtype} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} batch {batch}: current pick {pick} "
               f"({'%.1f us' % (t_pick * 1e3) if t_pick else 'not timed'}); fastest: "

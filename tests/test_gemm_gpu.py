@@ -629,9 +629,25 @@ def test_offline_tuner_emits_table_rows_for_small_shapes():
     rows = tune.tune(shapes, out)
     assert len(rows) == 3
     for row, s in zip(rows, shapes):
-        m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), ([\d.]+)f\},", row)
-        assert m and tuple(int(x) for x in m.groups()[:7]) == s[:7]
-        assert 0 <= int(m.group(8)) < G.num_configs(s[0]) and float(m.group(9)) > 0
+        m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+|ring_id\(\d, \d+\)|x16_id\(\d, \d+\)), ([\d.]+)f\},", row)
+        assert m and tuple(int(x) for x in m.groups()[:7]) == s[:7], row
+        assert float(m.group(9)) > 0
+        if m.group(8).isdigit():
+            assert 0 <= int(m.group(8)) < G.num_configs(s[0])
+    assert "FAILS" not in out.getvalue()
+    # the table syntax names the same config the id does
+    for dtype in (0, 1):
+        for cid in range(G.num_configs(dtype)):
+            d = G.config_info(dtype, cid)
+            t = tune.table_id(G, dtype, cid)
+            if "DTL1" not in d["name"]:
+                assert t == str(cid)
+            else:
+                fam, tile, split = re.match(r"(\w+)\((\d), (\d+)\)", t).groups()
+                assert (fam == "x16_id") == ("_ACC" in d["name"]) and int(split) == d["split_k"]
+                base = 50 if fam == "x16_id" else 30
+                ntile = 5 if fam == "x16_id" else 4
+                assert cid == base + int(tile) + ntile * [1, 2, 4, 8, 16].index(int(split))
 
 
 def test_automatic_pick_never_fails_on_its_own_choice():
