@@ -94,6 +94,12 @@ def build(force=False, verbose=True, jobs=None):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr[-4000:]}")
+    # a translation unit whose kernels silently failed to instantiate leaves the library with undefined symbols
+    import ctypes
+    try:
+        ctypes.CDLL(LIB, mode=getattr(os, "RTLD_NOW", 2))
+    except OSError as e:
+        raise RuntimeError(f"{LIB} does not load: {e}")
     if verbose:
         print(f"  linked {LIB}")
     return LIB

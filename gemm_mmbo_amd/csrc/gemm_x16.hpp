@@ -23,6 +23,24 @@ namespace mmbo {
 
 namespace x16 {
 
+// A work-group-uniform address as a scalar value (both halves through readfirstlane: the compiler then keeps what is
+// derived from it in scalar registers, where a buffer descriptor must live).
+__device__ __forceinline__ uint64_t uniform_address(const void *p)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// 16 bytes per lane from (uniform origin + the lane's 32-bit byte offset) straight into LDS at dst + lane * 16: a buffer
+// load whose descriptor holds the origin.  The descriptor's range is the 2 GiB a tile's span of an operand is limited
+// to, so it never clips; its last word is the raw 32-bit format of this chip family.
+__device__ __forceinline__ void direct_load16(uint64_t origin, uint32_t lane_offset, char *dst)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(origin), 0, 0x7fffffff, 0x00020000),
+                                             MMBO_LDS_PTR(dst), 16, lane_offset, 0, 0, 0);
+}
+
 using ring::lds_read_b128;
 using ring::lds_read_tr16_b64;
 using ring::static_for;
@@ -361,32 +379,30 @@ gemm_x16_kernel(const GemmArgs args)
 #pragma unroll
     for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here, backB);
 
-    // direct load number l (A's first, then B's) of slice s into ring buffer `buf`
-    auto issue_load = [&](auto L, const char *pa, const char *pb, char *dst) {
+    // The direct loads are buffer loads: the slice's origin sits in a scalar buffer descriptor (two scalar adds per slice
+    // and operand), the lane's part of the address is the 32-bit offset computed above, and no vector instruction is
+    // spent on addresses inside the slice loop (the global form takes a 64-bit address per lane: three 64-bit vector adds
+    // per pair of loads).  The descriptor's range is the 2 GiB a tile's span is limited to, so it never clips.
+    const uint64_t baseA = uniform_address(gA), baseB = uniform_address(gB);
+    auto slice_base = [&](uint64_t base, int64_t step, int s) { return base + (uint64_t)((int64_t)s * step); };
+    // direct load number l (A's first, then B's) of a slice (origins sa, sb) into ring buffer at dst
+    auto issue_load = [&](auto L, uint64_t sa, uint64_t sb, char *dst) {
         constexpr int l = decltype(L)::value;
-        if constexpr (l < TileA::LPW)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pa + offA[l]),
-                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + l) * 1024), 16, 0, 0);
-        else
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pb + offB[l - TileA::LPW]),
-                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024), 16, 0, 0);
+        if constexpr (l < TileA::LPW) direct_load16(sa, offA[l], dst + (wave * TileA::LPW + l) * 1024);
+        else direct_load16(sb, offB[l - TileA::LPW], dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024);
     };
     auto issue_slice = [&](int s, int buf) {
         char *dst = lds + buf * Cfg::SLICE_BYTES;
-        const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
-        static_for<BATCH>([&](auto L) { issue_load(L, pa, pb, dst); });
+        const uint64_t sa = slice_base(baseA, stepA, s), sb = slice_base(baseB, stepB, s);
+        static_for<BATCH>([&](auto L) { issue_load(L, sa, sb, dst); });
     };
 
     // load number i of operand OP (0 = A, 1 = B) of slice s into ring buffer b
     auto issue_op_load = [&](auto OP, auto I, int s, int b) {
         constexpr int op = decltype(OP)::value, i = decltype(I)::value;
         char *dst = lds + b * Cfg::SLICE_BYTES;
-        if constexpr (op == 0)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gA + (int64_t)s * stepA + offA[i]),
-                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + i) * 1024), 16, 0, 0);
-        else
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(gB + (int64_t)s * stepB + offB[i]),
-                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024), 16, 0, 0);
+        if constexpr (op == 0) direct_load16(slice_base(baseA, stepA, s), offA[i], dst + (wave * TileA::LPW + i) * 1024);
+        else direct_load16(slice_base(baseB, stepB, s), offB[i], dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024);
     };
 
     const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
@@ -423,7 +439,7 @@ gemm_x16_kernel(const GemmArgs args)
         const int pbuf = lbuf == 0 ? DEPTH - 1 : lbuf - 1;        // buffer of slice s+DEPTH-1
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         char *dst = lds + lbuf * Cfg::SLICE_BYTES;
-        const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
+        [[maybe_unused]] const uint64_t sa = slice_base(baseA, stepA, ls), sb = slice_base(baseB, stepB, ls);
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // boustrophedon over the FM x FN blocks: consecutive MFMAs share one operand register, also at the row
@@ -459,7 +475,7 @@ gemm_x16_kernel(const GemmArgs args)
                 static_for<l1 - l0>([&](auto LL) {
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < BATCH) {
-                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, pa, pb, dst);
+                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, sa, sb, dst);
                     }
                 });
             }
