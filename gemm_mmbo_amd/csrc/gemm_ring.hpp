@@ -6,7 +6,8 @@
 //
 // The reference's recipe (src/gemm/ref/Kernels.cpp:412-747: global prefetch ahead of use, LDS multi-buffer,
 // LDS->register prefetch of the next k step while the current one is multiplied) mapped onto CDNA4:
-//   - global -> LDS: global_load_lds_dwordx4; no register staging, no LDS write instructions.  Each lane
+//   - global -> LDS: buffer_load_dwordx4 ... lds (the slice's origin in a scalar descriptor, a 32-bit offset per lane);
+//     no register staging, no LDS write instructions, no vector address arithmetic in the loop.  Each lane
 //     fetches the 16-byte chunk whose XOR-swizzled LDS slot is (wave, instruction, lane); the swizzle removes
 //     the bank conflicts that padding would (a direct load writes 1 KB contiguously, so rows cannot be padded).
 //   - measured on MI355X, a batch of direct loads takes about 3,000 clocks to land when all 256 CUs stream,
@@ -63,6 +64,25 @@ __device__ __forceinline__ uint32_t lds_read_b32(uint32_t addr)
     uint32_t r;
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
     return r;
+}
+
+// A work-group-uniform address as a scalar value (both halves through readfirstlane: the compiler then keeps what is
+// derived from it in scalar registers, where a buffer descriptor must live).
+__device__ __forceinline__ uint64_t uniform_address(const void *p)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// 16 bytes per lane from (uniform origin + the lane's 32-bit byte offset) straight into LDS at dst + lane * 16: a buffer
+// load whose descriptor holds the origin.  The descriptor's range is the 2 GiB a tile's span of an operand is limited
+// to, so it never clips; its last word is the raw 32-bit format of this chip family.  (The global form of the same load
+// takes a 64-bit address per lane: three 64-bit vector adds per pair of loads inside the slice loop.)
+__device__ __forceinline__ void direct_load16(uint64_t origin, uint32_t lane_offset, char *dst)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(origin), 0, 0x7fffffff, 0x00020000),
+                                             MMBO_LDS_PTR(dst), 16, lane_offset, 0, 0, 0);
 }
 
 // One operand tile of one slice: R rows x BK along k = R * 64 bytes, loaded by NW wavefronts.
@@ -241,18 +261,15 @@ gemm_ring_kernel(const GemmArgs args)
 #pragma unroll
     for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb);
 
+    const uint64_t baseA = uniform_address(gA), baseB = uniform_address(gB);
     // slice s goes to ring buffer s % DEPTH; `buf` is that index, kept by the caller
     auto issue_slice = [&](int s, int buf) {
         char *dst = lds + buf * Cfg::SLICE_BYTES;
-        const char *pa = gA + (int64_t)s * stepA, *pb = gB + (int64_t)s * stepB;
+        const uint64_t sa = baseA + (uint64_t)((int64_t)s * stepA), sb = baseB + (uint64_t)((int64_t)s * stepB);
 #pragma unroll
-        for (int i = 0; i < TileA::LPW; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pa + offA[i]),
-                                             MMBO_LDS_PTR(dst + (wave * TileA::LPW + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < TileA::LPW; ++i) direct_load16(sa, offA[i], dst + (wave * TileA::LPW + i) * 1024);
 #pragma unroll
-        for (int i = 0; i < TileB::LPW; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(pb + offB[i]),
-                                             MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < TileB::LPW; ++i) direct_load16(sb, offB[i], dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024);
     };
 
     const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
@@ -288,7 +305,7 @@ gemm_ring_kernel(const GemmArgs args)
         constexpr bool always = decltype(ALWAYS)::value;          // steady state: every slice issues its loads, no flag test
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         char *dst = lds + lbuf * Cfg::SLICE_BYTES;
-        const char *pa = gA + (int64_t)ls * stepA, *pb = gB + (int64_t)ls * stepB;
+        const uint64_t sa = baseA + (uint64_t)((int64_t)ls * stepA), sb = baseB + (uint64_t)((int64_t)ls * stepB);
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // consecutive MFMAs go to different accumulators
@@ -319,14 +336,8 @@ gemm_ring_kernel(const GemmArgs args)
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < BATCH) {
                         if (always || load) {
-                            if constexpr (l < TileA::LPW)
-                                __builtin_amdgcn_global_load_lds(
-                                    (const __attribute__((address_space(1))) void *)(pa + offA[l]),
-                                    MMBO_LDS_PTR(dst + (wave * TileA::LPW + l) * 1024), 16, 0, 0);
-                            else
-                                __builtin_amdgcn_global_load_lds(
-                                    (const __attribute__((address_space(1))) void *)(pb + offB[l - TileA::LPW]),
-                                    MMBO_LDS_PTR(dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024), 16, 0, 0);
+                            if constexpr (l < TileA::LPW) direct_load16(sa, offA[l], dst + (wave * TileA::LPW + l) * 1024);
+                            else direct_load16(sb, offB[l - TileA::LPW], dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024);
                         }
                     }
                 });

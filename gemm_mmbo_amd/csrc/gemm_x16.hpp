@@ -23,27 +23,11 @@ namespace mmbo {
 
 namespace x16 {
 
-// A work-group-uniform address as a scalar value (both halves through readfirstlane: the compiler then keeps what is
-// derived from it in scalar registers, where a buffer descriptor must live).
-__device__ __forceinline__ uint64_t uniform_address(const void *p)
-{
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return ((uint64_t)hi << 32) | lo;
-}
-
-// 16 bytes per lane from (uniform origin + the lane's 32-bit byte offset) straight into LDS at dst + lane * 16: a buffer
-// load whose descriptor holds the origin.  The descriptor's range is the 2 GiB a tile's span of an operand is limited
-// to, so it never clips; its last word is the raw 32-bit format of this chip family.
-__device__ __forceinline__ void direct_load16(uint64_t origin, uint32_t lane_offset, char *dst)
-{
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(origin), 0, 0x7fffffff, 0x00020000),
-                                             MMBO_LDS_PTR(dst), 16, lane_offset, 0, 0, 0);
-}
-
+using ring::direct_load16;
 using ring::lds_read_b128;
 using ring::lds_read_tr16_b64;
 using ring::static_for;
+using ring::uniform_address;
 
 #define MMBO_AGPR_0_63 \
     "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15" , \
@@ -379,10 +363,9 @@ gemm_x16_kernel(const GemmArgs args)
 #pragma unroll
     for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here, backB);
 
-    // The direct loads are buffer loads: the slice's origin sits in a scalar buffer descriptor (two scalar adds per slice
-    // and operand), the lane's part of the address is the 32-bit offset computed above, and no vector instruction is
-    // spent on addresses inside the slice loop (the global form takes a 64-bit address per lane: three 64-bit vector adds
-    // per pair of loads).  The descriptor's range is the 2 GiB a tile's span is limited to, so it never clips.
+    // The direct loads are buffer loads (ring::direct_load16): the slice's origin sits in a scalar buffer descriptor (two
+    // scalar adds per slice and operand), the lane's part of the address is the 32-bit offset computed above, and no
+    // vector instruction is spent on addresses inside the slice loop.
     const uint64_t baseA = uniform_address(gA), baseB = uniform_address(gB);
     auto slice_base = [&](uint64_t base, int64_t step, int s) { return base + (uint64_t)((int64_t)s * step); };
     // direct load number l (A's first, then B's) of a slice (origins sa, sb) into ring buffer at dst
