@@ -75,14 +75,39 @@ __device__ __forceinline__ uint64_t uniform_address(const void *p)
     return ((uint64_t)hi << 32) | lo;
 }
 
-// 16 bytes per lane from (uniform origin + the lane's 32-bit byte offset) straight into LDS at dst + lane * 16: a buffer
-// load whose descriptor holds the origin.  The descriptor's range is the 2 GiB a tile's span of an operand is limited
-// to, so it never clips; its last word is the raw 32-bit format of this chip family.  (The global form of the same load
-// takes a 64-bit address per lane: three 64-bit vector adds per pair of loads inside the slice loop.)
-__device__ __forceinline__ void direct_load16(uint64_t origin, uint32_t lane_offset, char *dst)
+// The direct loads are buffer loads that write LDS (buffer_load_dwordx4 ... lds): 16 bytes per lane from
+//     descriptor origin + scalar offset + the lane's 32-bit byte offset      to      LDS at M0 + lane * 16.
+// An operand's descriptor lives in four scalar registers and is that operand's cursor: its origin is the next slice to be
+// requested and moves on by two scalar adds per slice; the lane offsets never change.  So the slice loop spends no
+// vector instruction on addresses (the global form of the load takes a 64-bit address per lane: three 64-bit vector adds
+// per pair of loads), and a load is three instructions in all -- M0, the wait state the hardware wants after a write to
+// M0, the load -- written as one asm statement so that nothing else lands between the MFMAs around it.  The statement
+// leaves M0 changed without saying so (the compiler refuses M0 in a clobber list): these kernels contain no other
+// instruction that reads M0, which tests/test_kernel_asm.py checks on the generated assembly.
+// The descriptor's range is the 2 GiB a tile's span of an operand is limited to, so it never clips; its last word is the
+// raw 32-bit format of this chip family.
+__device__ __forceinline__ u32x4 slice_cursor(uint64_t origin)
 {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(__builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(origin), 0, 0x7fffffff, 0x00020000),
-                                             MMBO_LDS_PTR(dst), 16, lane_offset, 0, 0, 0);
+    return u32x4{(uint32_t)origin, (uint32_t)(origin >> 32) & 0xffffu, 0x7fffffffu, 0x00020000u};
+}
+__device__ __forceinline__ void advance(u32x4 &cursor, uint64_t bytes)
+{
+    const uint64_t o = (((uint64_t)cursor[1] << 32) | cursor[0]) + bytes;       // (bits 48..63 of the second word stay zero)
+    cursor[0] = (uint32_t)o;
+    cursor[1] = (uint32_t)(o >> 32);
+}
+// lds_addr: work-group-uniform LDS byte address.  AHEAD = false: the slice at the cursor; true: the slice `step` bytes
+// further (step < 2 GiB by the tile-span limit).  (M0 is written with s_mov, which leaves the condition code alone: the
+// statement then writes nothing the compiler knows of, and two of them in a row are not padded apart.)
+template <bool AHEAD>
+__device__ __forceinline__ void direct_load16(const u32x4 &cursor, uint32_t step, uint32_t lane_offset, uint32_t lds_addr)
+{
+    if constexpr (AHEAD)
+        asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                     :: "v"(lane_offset), "s"(cursor), "s"(step), "s"(lds_addr) : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
+                     :: "v"(lane_offset), "s"(cursor), "s"(lds_addr) : "memory");
 }
 
 // One operand tile of one slice: R rows x BK along k = R * 64 bytes, loaded by NW wavefronts.
@@ -261,15 +286,17 @@ gemm_ring_kernel(const GemmArgs args)
 #pragma unroll
     for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb);
 
-    const uint64_t baseA = uniform_address(gA), baseB = uniform_address(gB);
-    // slice s goes to ring buffer s % DEPTH; `buf` is that index, kept by the caller
-    auto issue_slice = [&](int s, int buf) {
-        char *dst = lds + buf * Cfg::SLICE_BYTES;
-        const uint64_t sa = baseA + (uint64_t)((int64_t)s * stepA), sb = baseB + (uint64_t)((int64_t)s * stepB);
-#pragma unroll
-        for (int i = 0; i < TileA::LPW; ++i) direct_load16(sa, offA[i], dst + (wave * TileA::LPW + i) * 1024);
-#pragma unroll
-        for (int i = 0; i < TileB::LPW; ++i) direct_load16(sb, offB[i], dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024);
+    // cursors of the two operands: the next slice to be requested (slices are requested in order, one per iteration)
+    u32x4 curA = slice_cursor(uniform_address(gA)), curB = slice_cursor(uniform_address(gB));
+    const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
+    const uint32_t ldsA = lds_base + wave * TileA::LPW * 1024, ldsB = lds_base + TileA::BYTES + wave * TileB::LPW * 1024;
+    // the next slice goes to ring buffer `buf` (slice s to buffer s % DEPTH, kept by the caller)
+    auto issue_slice = [&](int buf) {
+        const uint32_t bo = buf * Cfg::SLICE_BYTES;
+        static_for<TileA::LPW>([&](auto I) { direct_load16<false>(curA, 0u, offA[decltype(I)::value], ldsA + bo + decltype(I)::value * 1024); });
+        static_for<TileB::LPW>([&](auto I) { direct_load16<false>(curB, 0u, offB[decltype(I)::value], ldsB + bo + decltype(I)::value * 1024); });
+        advance(curA, (uint64_t)stepA);
+        advance(curB, (uint64_t)stepB);
     };
 
     const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
@@ -284,7 +311,6 @@ gemm_ring_kernel(const GemmArgs args)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
@@ -301,11 +327,10 @@ gemm_ring_kernel(const GemmArgs args)
     // slice has the larger the exposed share: measured on fp32 4096 x 128 x 4096, reads spread over the whole slice
     // cost 10 us on top of 35 us of MFMAs.
     constexpr int READ_SPAN = Cfg::NW > 4 ? NMFMA : (NMFMA >= 32 ? NMFMA * 3 / 4 : NMFMA / 2);
-    auto mfma_and_read = [&](auto ALWAYS, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int ls, int lbuf) {
+    auto mfma_and_read = [&](auto ALWAYS, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load, int lbuf) {
         constexpr bool always = decltype(ALWAYS)::value;          // steady state: every slice issues its loads, no flag test
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
-        char *dst = lds + lbuf * Cfg::SLICE_BYTES;
-        const uint64_t sa = baseA + (uint64_t)((int64_t)ls * stepA), sb = baseB + (uint64_t)((int64_t)ls * stepB);
+        const uint32_t dstA = ldsA + lbuf * Cfg::SLICE_BYTES, dstB = ldsB + lbuf * Cfg::SLICE_BYTES;
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // consecutive MFMAs go to different accumulators
@@ -336,14 +361,18 @@ gemm_ring_kernel(const GemmArgs args)
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < BATCH) {
                         if (always || load) {
-                            if constexpr (l < TileA::LPW) direct_load16(sa, offA[l], dst + (wave * TileA::LPW + l) * 1024);
-                            else direct_load16(sb, offB[l - TileA::LPW], dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024);
+                            if constexpr (l < TileA::LPW) direct_load16<false>(curA, 0u, offA[l], dstA + l * 1024);
+                            else direct_load16<false>(curB, 0u, offB[l - TileA::LPW], dstB + (l - TileA::LPW) * 1024);
                         }
                     }
                 });
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        if (always || load) {                                     // the cursors move on to the slice after the one just requested
+            advance(curA, (uint64_t)stepA);
+            advance(curB, (uint64_t)stepB);
+        }
     };
 #define MMBO_BARRIER()                           \
     do {                                         \
@@ -363,7 +392,7 @@ gemm_ring_kernel(const GemmArgs args)
     // tail stops issuing, the wait is for everything.
 #pragma unroll
     for (int s = 0; s < DEPTH; ++s)
-        if (s < n_slice) issue_slice(s, s);
+        if (s < n_slice) issue_slice(s);
     if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
     MMBO_BARRIER();                                                  // slice 0 resident
     read_slice(fa[0], fb[0], 0);
@@ -376,7 +405,7 @@ gemm_ring_kernel(const GemmArgs args)
     // smallest fp16 tile the tests and branches were a third of the instructions a wavefront issued per slice)
     auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
         const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-        mfma_and_read(std::true_type{}, ca, cb, na, nb, nbuf, true, s + DEPTH, buf);
+        mfma_and_read(std::true_type{}, ca, cb, na, nb, nbuf, true, buf);
         MMBO_WAIT_LGKM0();
         MMBO_WAIT_VM(BATCH * (DEPTH - 2));
         MMBO_BARRIER();
@@ -387,7 +416,7 @@ gemm_ring_kernel(const GemmArgs args)
         const bool steady = s + DEPTH < n_slice;
         // (the last slice reads a stale buffer into the unused register set: harmless, and it keeps the
         // interleaved block free of divergent control flow)
-        mfma_and_read(std::false_type{}, ca, cb, na, nb, nbuf, steady, s + DEPTH, buf);
+        mfma_and_read(std::false_type{}, ca, cb, na, nb, nbuf, steady, buf);
         MMBO_WAIT_LGKM0();
         if (steady) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();

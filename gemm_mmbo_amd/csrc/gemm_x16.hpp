@@ -23,9 +23,11 @@ namespace mmbo {
 
 namespace x16 {
 
+using ring::advance;
 using ring::direct_load16;
 using ring::lds_read_b128;
 using ring::lds_read_tr16_b64;
+using ring::slice_cursor;
 using ring::static_for;
 using ring::uniform_address;
 
@@ -363,29 +365,38 @@ gemm_x16_kernel(const GemmArgs args)
 #pragma unroll
     for (int i = 0; i < TileB::LPW; ++i) offB[i] = TileB::load_goff(wave, lane, i, ldb, n_here, backB);
 
-    // The direct loads are buffer loads (ring::direct_load16): the slice's origin sits in a scalar buffer descriptor (two
-    // scalar adds per slice and operand), the lane's part of the address is the 32-bit offset computed above, and no
-    // vector instruction is spent on addresses inside the slice loop.
-    const uint64_t baseA = uniform_address(gA), baseB = uniform_address(gB);
-    auto slice_base = [&](uint64_t base, int64_t step, int s) { return base + (uint64_t)((int64_t)s * step); };
-    // direct load number l (A's first, then B's) of a slice (origins sa, sb) into ring buffer at dst
-    auto issue_load = [&](auto L, uint64_t sa, uint64_t sb, char *dst) {
-        constexpr int l = decltype(L)::value;
-        if constexpr (l < TileA::LPW) direct_load16(sa, offA[l], dst + (wave * TileA::LPW + l) * 1024);
-        else direct_load16(sb, offB[l - TileA::LPW], dst + TileA::BYTES + (wave * TileB::LPW + l - TileA::LPW) * 1024);
-    };
-    auto issue_slice = [&](int s, int buf) {
-        char *dst = lds + buf * Cfg::SLICE_BYTES;
-        const uint64_t sa = slice_base(baseA, stepA, s), sb = slice_base(baseB, stepB, s);
-        static_for<BATCH>([&](auto L) { issue_load(L, sa, sb, dst); });
-    };
-
-    // load number i of operand OP (0 = A, 1 = B) of slice s into ring buffer b
-    auto issue_op_load = [&](auto OP, auto I, int s, int b) {
+    // The direct loads (ring::direct_load16): each operand has a cursor, a buffer descriptor in scalar registers whose
+    // origin is the next slice to be requested; the lane's part of the address is the 32-bit offset computed above.
+    // Slices are requested in order, so a request is "the slice at the cursor" (or, in paired mode, also the one after
+    // it), and the cursor then moves on.
+    u32x4 curA = slice_cursor(uniform_address(gA)), curB = slice_cursor(uniform_address(gB));
+    const uint32_t stepA32 = (uint32_t)stepA, stepB32 = (uint32_t)stepB;       // below 2 GiB: the tile-span limit
+    const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
+    const uint32_t ldsA = lds_base + wave * TileA::LPW * 1024, ldsB = lds_base + TileA::BYTES + wave * TileB::LPW * 1024;
+    // load number i of operand OP (0 = A, 1 = B), of the slice at the cursor (AHEAD = false) or the one after it, to
+    // dst = this wavefront's first LDS destination of that operand in the ring buffer the slice goes to (op_dst)
+    auto op_dst = [&](auto OP, int b) { return (decltype(OP)::value == 0 ? ldsA : ldsB) + (uint32_t)b * Cfg::SLICE_BYTES; };
+    auto issue_op_load = [&](auto OP, auto I, auto AHEAD, uint32_t dst) {
         constexpr int op = decltype(OP)::value, i = decltype(I)::value;
-        char *dst = lds + b * Cfg::SLICE_BYTES;
-        if constexpr (op == 0) direct_load16(slice_base(baseA, stepA, s), offA[i], dst + (wave * TileA::LPW + i) * 1024);
-        else direct_load16(slice_base(baseB, stepB, s), offB[i], dst + TileA::BYTES + (wave * TileB::LPW + i) * 1024);
+        constexpr bool ahead = decltype(AHEAD)::value;
+        if constexpr (op == 0) direct_load16<ahead>(curA, stepA32, offA[i], dst + i * 1024);
+        else direct_load16<ahead>(curB, stepB32, offB[i], dst + i * 1024);
+    };
+    auto advance_op = [&](auto OP, int slices) {
+        if constexpr (decltype(OP)::value == 0) advance(curA, (uint64_t)stepA * slices);
+        else advance(curB, (uint64_t)stepB * slices);
+    };
+    // direct load number l (A's first, then B's) of the slices at the two cursors into ring buffer `buf`
+    auto issue_load = [&](auto L, uint32_t dst_a, uint32_t dst_b) {
+        constexpr int l = decltype(L)::value;
+        if constexpr (l < TileA::LPW) issue_op_load(std::integral_constant<int, 0>{}, L, std::false_type{}, dst_a);
+        else issue_op_load(std::integral_constant<int, 1>{}, std::integral_constant<int, l - TileA::LPW>{}, std::false_type{}, dst_b);
+    };
+    auto issue_slice = [&](int buf) {
+        const uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, buf), dst_b = op_dst(std::integral_constant<int, 1>{}, buf);
+        static_for<BATCH>([&](auto L) { issue_load(L, dst_a, dst_b); });
+        advance(curA, (uint64_t)stepA);
+        advance(curB, (uint64_t)stepB);
     };
 
     const typename FragA::Addr adA = FragA::make_addr(lane, wm * Cfg::TM);
@@ -394,7 +405,6 @@ gemm_x16_kernel(const GemmArgs args)
     FragB fb[2];
     acc_zero<NACC>();
 
-    const uint32_t lds_base = (uint32_t)(uintptr_t)MMBO_LDS_PTR(lds);
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
@@ -414,15 +424,19 @@ gemm_x16_kernel(const GemmArgs args)
     // (measured: half-line requests stream at 35-52 B/clk/CU from L2, whole lines at 72-91).  `load` / `load2`
     // say whether the first / second slice of the pair exists.
     auto mfma_and_read = [&](auto LOAD, auto PAR, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load,
-                             bool load2, int ls, int lbuf) {
+                             bool load2, int lbuf) {
         constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load` (and `load2`)
         constexpr int par = decltype(PAR)::value;
         constexpr int opn = par ^ EVEN_OP;                         // paired mode: the operand this iteration fetches
         constexpr int LOP = opn == 0 ? TileA::LPW : TileB::LPW;   // and its loads per slice
         const int pbuf = lbuf == 0 ? DEPTH - 1 : lbuf - 1;        // buffer of slice s+DEPTH-1
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
-        char *dst = lds + lbuf * Cfg::SLICE_BYTES;
-        [[maybe_unused]] const uint64_t sa = slice_base(baseA, stepA, ls), sb = slice_base(baseB, stepB, ls);
+        // LDS destinations of this iteration's loads, worked out here, once (the empty asm pins them to scalar registers
+        // at this point: otherwise the compiler recomputes them next to every load, between two MFMAs)
+        uint32_t dst_x0 = op_dst(std::integral_constant<int, opn>{}, pbuf), dst_x1 = op_dst(std::integral_constant<int, opn>{}, lbuf);
+        uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, lbuf), dst_b = op_dst(std::integral_constant<int, 1>{}, lbuf);
+        if constexpr (load_mode != 0 && PAIR) asm volatile("" : "+s"(dst_x0), "+s"(dst_x1));
+        if constexpr (load_mode != 0 && !PAIR) asm volatile("" : "+s"(dst_a), "+s"(dst_b));
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // boustrophedon over the FM x FN blocks: consecutive MFMAs share one operand register, also at the row
@@ -443,12 +457,21 @@ gemm_x16_kernel(const GemmArgs args)
                 });
             }
             if constexpr (load_mode != 0 && PAIR) {
+                // load l of the first slice of the pair goes out after MFMA number (2l+1) * NMFMA / (2 * LOP), the load of the
+                // second slice that shares its memory lines one MFMA later: three instructions each, which fit between two MFMAs
                 constexpr int l0 = (2 * LOP * m + NMFMA) / (2 * NMFMA), l1 = (2 * LOP * (m + 1) + NMFMA) / (2 * NMFMA);
+                constexpr int p0 = m == 0 ? 0 : (2 * LOP * (m - 1) + NMFMA) / (2 * NMFMA);
+                static_assert(m + 1 < NMFMA || l1 - l0 == 0 || l0 >= LOP, "the last MFMA slot cannot start a pair of loads");
+                static_for<l0 - p0>([&](auto LL) {
+                    constexpr int l = p0 + decltype(LL)::value;
+                    if constexpr (l < LOP) {
+                        if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::true_type{}, dst_x1);
+                    }
+                });
                 static_for<l1 - l0>([&](auto LL) {
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < LOP) {
-                        if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, ls - 1, pbuf);
-                        if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, ls, lbuf);
+                        if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::false_type{}, dst_x0);
                     }
                 });
             }
@@ -458,12 +481,18 @@ gemm_x16_kernel(const GemmArgs args)
                 static_for<l1 - l0>([&](auto LL) {
                     constexpr int l = l0 + decltype(LL)::value;
                     if constexpr (l < BATCH) {
-                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, sa, sb, dst);
+                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b);
                     }
                 });
             }
             __builtin_amdgcn_sched_barrier(0);
         });
+        // the cursors move past what this iteration requested (past the end of k in the last iterations: never used again)
+        if constexpr (load_mode != 0 && PAIR) advance_op(std::integral_constant<int, opn>{}, 2);
+        if constexpr (load_mode != 0 && !PAIR) {
+            advance(curA, (uint64_t)stepA);
+            advance(curB, (uint64_t)stepB);
+        }
     };
 #define MMBO_BARRIER()                           \
     do {                                         \
@@ -485,7 +514,7 @@ gemm_x16_kernel(const GemmArgs args)
     if constexpr (!PAIR) {
 #pragma unroll
         for (int q = 0; q < DEPTH; ++q)
-            if (q < n_slice) issue_slice(q, q);
+            if (q < n_slice) issue_slice(q);
         if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slice 0 resident
         read_slice(fa[0], fb[0], 0);
@@ -496,7 +525,7 @@ gemm_x16_kernel(const GemmArgs args)
         // steady state: every slice issues loads, no flag tests inside the MFMA stream
         auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-            mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
+            mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, buf);
             MMBO_WAIT_LGKM0();
             MMBO_WAIT_VM(BATCH * (DEPTH - 2));
             MMBO_BARRIER();
@@ -507,7 +536,7 @@ gemm_x16_kernel(const GemmArgs args)
         auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH < n_slice;
-            mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, s + DEPTH, buf);
+            mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, buf);
             MMBO_WAIT_LGKM0();
             if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
             MMBO_BARRIER();
@@ -531,8 +560,12 @@ gemm_x16_kernel(const GemmArgs args)
 #pragma unroll
         for (int q = 0; q < DEPTH; ++q) {
             if (q < n_slice) {
-                if (q < DEPTH - 1) static_for<LA>([&](auto I) { issue_op_load(OPX, I, q, q); });
-                static_for<LB>([&](auto I) { issue_op_load(OPY, I, q, q); });
+                if (q < DEPTH - 1) {
+                    static_for<LA>([&](auto I) { issue_op_load(OPX, I, std::false_type{}, op_dst(OPX, q)); });
+                    advance_op(OPX, 1);
+                }
+                static_for<LB>([&](auto I) { issue_op_load(OPY, I, std::false_type{}, op_dst(OPY, q)); });
+                advance_op(OPY, 1);
             }
         }
         constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
@@ -550,7 +583,7 @@ gemm_x16_kernel(const GemmArgs args)
             constexpr int KEEP = own * ((DEPTH - 3 + 1) / 2) + other * ((DEPTH - 3) / 2);
             static_assert(KEEP < 64, "more loads in flight than vmcnt can count");
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-            mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, s + DEPTH, buf);
+            mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, buf);
             MMBO_WAIT_LGKM0();
             MMBO_WAIT_VM(KEEP);
             MMBO_BARRIER();
@@ -565,7 +598,7 @@ gemm_x16_kernel(const GemmArgs args)
             static_assert(LA % G == 0 && LB % G == 0, "loads per slice of one operand must divide the other's");
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
-            mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, s + DEPTH, buf);
+            mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf);
             MMBO_WAIT_LGKM0();
             const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP;
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
