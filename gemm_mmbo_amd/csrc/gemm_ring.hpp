@@ -110,6 +110,17 @@ __device__ __forceinline__ void direct_load16(const u32x4 &cursor, uint32_t step
                      :: "v"(lane_offset), "s"(cursor), "s"(lds_addr) : "memory");
 }
 
+// The same load in two statements, for callers that put another asm statement (an MFMA) between them: that statement is
+// then the wait state between the write to M0 and the load, and the s_nop is saved.  The caller guarantees that at least
+// one instruction it controls sits between the two.
+__device__ __forceinline__ void set_lds_destination(uint32_t lds_addr) { asm volatile("s_mov_b32 m0, %0" :: "s"(lds_addr)); }
+template <bool AHEAD>
+__device__ __forceinline__ void direct_load16_to_destination(const u32x4 &cursor, uint32_t step, uint32_t lane_offset)
+{
+    if constexpr (AHEAD) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" :: "v"(lane_offset), "s"(cursor), "s"(step) : "memory");
+    else asm volatile("buffer_load_dwordx4 %0, %1, 0 offen lds" :: "v"(lane_offset), "s"(cursor) : "memory");
+}
+
 // One operand tile of one slice: R rows x BK along k = R * 64 bytes, loaded by NW wavefronts.
 //   KC (source contiguous along k): LDS row r = its 64 bytes = 4 chunks of 16 B; chunk c sits at position
 //     c ^ ((r >> 2) & 3), so 16 consecutive rows reading the same logical chunk cover all sixteen 16-byte

@@ -25,8 +25,10 @@ namespace x16 {
 
 using ring::advance;
 using ring::direct_load16;
+using ring::direct_load16_to_destination;
 using ring::lds_read_b128;
 using ring::lds_read_tr16_b64;
+using ring::set_lds_destination;
 using ring::slice_cursor;
 using ring::static_for;
 using ring::uniform_address;
@@ -272,6 +274,14 @@ struct Frags {
     }
 };
 
+// How many of a slice's `loads` direct loads have gone out before MFMA slot `slot` of `slots`: load l goes out after MFMA
+// number (2l+1) * slots / (2 * loads), evenly spaced, none first or last.
+constexpr int loads_before_slot(int loads, int slots, int slot)
+{
+    const int l = (2 * loads * slot + slots) / (2 * slots);
+    return l < loads ? l : loads;
+}
+
 }  // namespace x16
 
 template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH>
@@ -376,25 +386,30 @@ gemm_x16_kernel(const GemmArgs args)
     // load number i of operand OP (0 = A, 1 = B), of the slice at the cursor (AHEAD = false) or the one after it, to
     // dst = this wavefront's first LDS destination of that operand in the ring buffer the slice goes to (op_dst)
     auto op_dst = [&](auto OP, int b) { return (decltype(OP)::value == 0 ? ldsA : ldsB) + (uint32_t)b * Cfg::SLICE_BYTES; };
-    auto issue_op_load = [&](auto OP, auto I, auto AHEAD, uint32_t dst) {
+    auto issue_op_load = [&](auto OP, auto I, auto AHEAD, uint32_t dst, auto DESTINATION_SET) {
         constexpr int op = decltype(OP)::value, i = decltype(I)::value;
         constexpr bool ahead = decltype(AHEAD)::value;
-        if constexpr (op == 0) direct_load16<ahead>(curA, stepA32, offA[i], dst + i * 1024);
-        else direct_load16<ahead>(curB, stepB32, offB[i], dst + i * 1024);
+        if constexpr (decltype(DESTINATION_SET)::value) {           // M0 was written before the MFMA just issued
+            if constexpr (op == 0) direct_load16_to_destination<ahead>(curA, stepA32, offA[i]);
+            else direct_load16_to_destination<ahead>(curB, stepB32, offB[i]);
+        } else {
+            if constexpr (op == 0) direct_load16<ahead>(curA, stepA32, offA[i], dst + i * 1024);
+            else direct_load16<ahead>(curB, stepB32, offB[i], dst + i * 1024);
+        }
     };
     auto advance_op = [&](auto OP, int slices) {
         if constexpr (decltype(OP)::value == 0) advance(curA, (uint64_t)stepA * slices);
         else advance(curB, (uint64_t)stepB * slices);
     };
     // direct load number l (A's first, then B's) of the slices at the two cursors into ring buffer `buf`
-    auto issue_load = [&](auto L, uint32_t dst_a, uint32_t dst_b) {
+    auto issue_load = [&](auto L, uint32_t dst_a, uint32_t dst_b, auto DESTINATION_SET) {
         constexpr int l = decltype(L)::value;
-        if constexpr (l < TileA::LPW) issue_op_load(std::integral_constant<int, 0>{}, L, std::false_type{}, dst_a);
-        else issue_op_load(std::integral_constant<int, 1>{}, std::integral_constant<int, l - TileA::LPW>{}, std::false_type{}, dst_b);
+        if constexpr (l < TileA::LPW) issue_op_load(std::integral_constant<int, 0>{}, L, std::false_type{}, dst_a, DESTINATION_SET);
+        else issue_op_load(std::integral_constant<int, 1>{}, std::integral_constant<int, l - TileA::LPW>{}, std::false_type{}, dst_b, DESTINATION_SET);
     };
     auto issue_slice = [&](int buf) {
         const uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, buf), dst_b = op_dst(std::integral_constant<int, 1>{}, buf);
-        static_for<BATCH>([&](auto L) { issue_load(L, dst_a, dst_b); });
+        static_for<BATCH>([&](auto L) { issue_load(L, dst_a, dst_b, std::false_type{}); });
         advance(curA, (uint64_t)stepA);
         advance(curB, (uint64_t)stepB);
     };
@@ -444,10 +459,25 @@ gemm_x16_kernel(const GemmArgs args)
             // fp32 walks the blocks four times, once per k register, so an accumulator recurs every FM*FN MFMAs
             constexpr int tt = m / (FM * FN), ij = m % (FM * FN);
             constexpr int i = ij / FN, j = (i & 1) ? FN - 1 - ij % FN : ij % FN;
+            // The direct loads that go out after this MFMA (known at compile time).  Paired mode: load l of the first slice
+            // of the pair after MFMA number (2l+1) * NMFMA / (2 * LOP), the load of the second slice, which shares its memory
+            // lines, one MFMA later.  Unpaired: load l after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none
+            // first or last.  Where exactly one load follows the MFMA, its LDS destination goes into M0 BEFORE the MFMA and the
+            // load itself after it: the MFMA is the wait state a write to M0 needs, and the load costs two instructions.
+            constexpr int LIM = PAIR ? LOP : BATCH;
+            constexpr int l0 = loads_before_slot(LIM, NMFMA, m), l1 = loads_before_slot(LIM, NMFMA, m + 1),
+                          p0 = m == 0 ? 0 : loads_before_slot(LIM, NMFMA, m - 1);
+            constexpr int n_first = load_mode != 0 ? l1 - l0 : 0, n_second = (load_mode != 0 && PAIR) ? l0 - p0 : 0;
+            static_assert(!PAIR || m + 1 < NMFMA || n_first == 0, "the last MFMA slot cannot start a pair of loads");
+            constexpr bool single = n_first + n_second == 1;
+            if constexpr (single) {
+                if constexpr (n_second == 1) set_lds_destination(dst_x1 + p0 * 1024);
+                else if constexpr (PAIR) set_lds_destination(dst_x0 + l0 * 1024);
+                else if constexpr (l0 < TileA::LPW) set_lds_destination(dst_a + l0 * 1024);
+                else set_lds_destination(dst_b + (l0 - TileA::LPW) * 1024);
+            }
             if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
             else mfma_acc_f32<(i * FN + j) * 4, NACC>(ca.x[i][tt], cb.x[j][tt]);
-            // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
-            // pad the gap with an s_nop, which costs an issue slot like any other instruction)
             if constexpr (m < READ_SPAN) {
                 constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
                 static_for<r1 - r0>([&](auto RR) {
@@ -456,35 +486,21 @@ gemm_x16_kernel(const GemmArgs args)
                     else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
                 });
             }
-            if constexpr (load_mode != 0 && PAIR) {
-                // load l of the first slice of the pair goes out after MFMA number (2l+1) * NMFMA / (2 * LOP), the load of the
-                // second slice that shares its memory lines one MFMA later: three instructions each, which fit between two MFMAs
-                constexpr int l0 = (2 * LOP * m + NMFMA) / (2 * NMFMA), l1 = (2 * LOP * (m + 1) + NMFMA) / (2 * NMFMA);
-                constexpr int p0 = m == 0 ? 0 : (2 * LOP * (m - 1) + NMFMA) / (2 * NMFMA);
-                static_assert(m + 1 < NMFMA || l1 - l0 == 0 || l0 >= LOP, "the last MFMA slot cannot start a pair of loads");
-                static_for<l0 - p0>([&](auto LL) {
-                    constexpr int l = p0 + decltype(LL)::value;
-                    if constexpr (l < LOP) {
-                        if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::true_type{}, dst_x1);
-                    }
-                });
-                static_for<l1 - l0>([&](auto LL) {
-                    constexpr int l = l0 + decltype(LL)::value;
-                    if constexpr (l < LOP) {
-                        if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::false_type{}, dst_x0);
-                    }
-                });
-            }
-            if constexpr (load_mode != 0 && !PAIR) {
-                // load l goes out after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none first or last
-                constexpr int l0 = (2 * BATCH * m + NMFMA) / (2 * NMFMA), l1 = (2 * BATCH * (m + 1) + NMFMA) / (2 * NMFMA);
-                static_for<l1 - l0>([&](auto LL) {
-                    constexpr int l = l0 + decltype(LL)::value;
-                    if constexpr (l < BATCH) {
-                        if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b);
-                    }
-                });
-            }
+            constexpr std::bool_constant<single> DESTINATION_SET{};
+            static_for<n_second>([&](auto LL) {
+                constexpr int l = p0 + decltype(LL)::value;
+                if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::true_type{}, dst_x1, DESTINATION_SET);
+            });
+            static_for<n_first>([&](auto LL) {
+                constexpr int l = l0 + decltype(LL)::value;
+                if constexpr (PAIR) {
+                    if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::false_type{}, dst_x0, DESTINATION_SET);
+                } else {
+                    if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b, DESTINATION_SET);
+                }
+            });
+            // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
+            // pad the gap with an s_nop, which costs an issue slot like any other instruction)
             __builtin_amdgcn_sched_barrier(0);
         });
         // the cursors move past what this iteration requested (past the end of k in the last iterations: never used again)
@@ -561,10 +577,10 @@ gemm_x16_kernel(const GemmArgs args)
         for (int q = 0; q < DEPTH; ++q) {
             if (q < n_slice) {
                 if (q < DEPTH - 1) {
-                    static_for<LA>([&](auto I) { issue_op_load(OPX, I, std::false_type{}, op_dst(OPX, q)); });
+                    static_for<LA>([&](auto I) { issue_op_load(OPX, I, std::false_type{}, op_dst(OPX, q), std::false_type{}); });
                     advance_op(OPX, 1);
                 }
-                static_for<LB>([&](auto I) { issue_op_load(OPY, I, std::false_type{}, op_dst(OPY, q)); });
+                static_for<LB>([&](auto I) { issue_op_load(OPY, I, std::false_type{}, op_dst(OPY, q), std::false_type{}); });
                 advance_op(OPY, 1);
             }
         }

@@ -141,6 +141,44 @@ def test_no_register_is_touched_while_its_lds_read_is_in_flight(asm_files):
     assert checked >= 4 * (10 + 8)         # four transposes of every tile of both families, both element types
 
 
+def _compiler_generated(path):
+    """{kernel symbol: instruction lines the compiler generated itself}, i.e. everything outside the ;;#ASMSTART ... ;;#ASMEND
+    brackets the compiler puts around the text of an asm statement."""
+    lines = open(path).read().split("\n")
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_Z\w+:", l)]
+    out = {}
+    for n, i in enumerate(starts):
+        end = starts[n + 1] if n + 1 < len(starts) else len(lines)
+        body, inside = [], False
+        for l in lines[i + 1:end]:
+            t = l.strip()
+            if t.startswith(".amdhsa_kernel") or t.startswith(".section"):
+                break
+            if t.startswith(";;#ASMSTART"):
+                inside = True
+            elif t.startswith(";;#ASMEND"):
+                inside = False
+            elif not inside and t and not t.startswith(";") and not t.startswith(".") and not re.match(r"^\.?LBB\w+:", t):
+                body.append(t.split(";")[0].strip())
+        out[lines[i].split(":")[0]] = body
+    return out
+
+
+def test_nothing_but_the_direct_loads_touches_m0(asm_files):
+    """The direct loads set M0 (the LDS destination) inside their own asm statement and leave it changed without telling
+    the compiler, which refuses M0 in a clobber list.  That is only sound while the compiler keeps nothing in M0 itself:
+    no instruction it generated for these kernels may name M0."""
+    checked = 0
+    for path in asm_files:
+        for name, body in _compiler_generated(path).items():
+            bad = [t for t in body if re.search(r"\bm0\b", t)]
+            assert not bad, f"{name}: compiler-generated use of m0: {bad[:3]}"
+            checked += 1
+        text = open(path).read()
+        assert "buffer_load_dwordx4" in text and " lds" in text        # the asm statements are there (and inside brackets)
+    assert checked >= 4 * (10 + 8)
+
+
 def _main_loops(body):
     """(first, last) instruction index of the innermost backward-branch ranges that hold MFMAs but neither a store to
     global memory nor the zeroing of an accumulator: the steady-state slice loops.  (The loop over the tiles of a resident
