@@ -275,7 +275,11 @@ gemm_ring_kernel(const GemmArgs args)
     uint32_t wg0, wg1, tile_id, zb, nxcd;
     work_of_block(args, blockIdx.x, blockIdx.z, tile_id, zb, nxcd);
     wg_remap(tile_id, args.nwg0, args.nwg1, args.wgm, nxcd, wg0, wg1);
-    const uint32_t split = zb / args.batch, batch = zb % args.batch;
+    wg0 = __builtin_amdgcn_readfirstlane(wg0);
+    wg1 = __builtin_amdgcn_readfirstlane(wg1);
+    // (the division runs on the vector unit: back to scalar registers, so that what follows from it -- the k range, the
+    // slice count, the loop test -- stays scalar as well)
+    const uint32_t split = __builtin_amdgcn_readfirstlane(zb / args.batch), batch = __builtin_amdgcn_readfirstlane(zb % args.batch);
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
     const uint32_t lda = args.lda, ldb = args.ldb;
     const uint32_t k_begin = split * args.k_per_split;

@@ -346,7 +346,9 @@ gemm_x16_kernel(const GemmArgs args)
     wg0 = __builtin_amdgcn_readfirstlane(wg0);
     wg1 = __builtin_amdgcn_readfirstlane(wg1);
     zb = __builtin_amdgcn_readfirstlane(zb);
-    const uint32_t split = zb / args.batch, batch = zb % args.batch;
+    // (the division runs on the vector unit: back to scalar registers, so that what follows from it -- the k range, the
+    // slice count, the loop test -- stays scalar as well)
+    const uint32_t split = __builtin_amdgcn_readfirstlane(zb / args.batch), batch = __builtin_amdgcn_readfirstlane(zb % args.batch);
     const uint32_t row0 = wg0 * BM, col0 = wg1 * BN;
     const uint32_t lda = args.lda, ldb = args.ldb;
     const uint32_t k_begin = split * args.k_per_split;
