@@ -226,7 +226,8 @@ struct Frags {
     static constexpr int NOPS = F * RPF;
     u32x4 x[F];
 
-    struct Addr { uint32_t a[KC ? 1 : F]; };
+    static constexpr int NADDR = KC ? 1 : F;                         // distinct read addresses per slice
+    struct Addr { uint32_t a[NADDR]; };
 
     __device__ static inline Addr make_addr(int lane, int r0)
     {
@@ -254,19 +255,28 @@ struct Frags {
         return ad;
     }
 
+    // Read number OP of a slice takes the address tile + ad.a[address_index(OP)] plus a constant; consecutive reads
+    // share addresses, and first_use(OP) says whether OP is the first to use its one.
+    static constexpr int address_index(int op) { return KC ? 0 : op / RPF; }
+    static constexpr bool first_use(int op) { return KC ? op == 0 : op % RPF == 0; }
     template <int OP>
-    __device__ __forceinline__ void read_op(uint32_t tile, const Addr &ad)
+    __device__ __forceinline__ void read_op_at(uint32_t address)
     {
         constexpr int f = OP / RPF, h = OP % RPF;
         if constexpr (KC) {
-            x[f] = lds_read_b128<f * 16 * 64>(tile + ad.a[0]);
+            x[f] = lds_read_b128<f * 16 * 64>(address);
         } else if constexpr (ESZ == 4) {
-            x[f][h] = ring::lds_read_b32<h * T::ROW_BYTES>(tile + ad.a[f]);
+            x[f][h] = ring::lds_read_b32<h * T::ROW_BYTES>(address);
         } else {
-            u32x2 v = lds_read_tr16_b64<h * 4 * T::ROW_BYTES>(tile + ad.a[f]);
+            u32x2 v = lds_read_tr16_b64<h * 4 * T::ROW_BYTES>(address);
             x[f][2 * h] = v[0];
             x[f][2 * h + 1] = v[1];
         }
+    }
+    template <int OP>
+    __device__ __forceinline__ void read_op(uint32_t tile, const Addr &ad)
+    {
+        read_op_at<OP>(tile + ad.a[address_index(OP)]);
     }
     __device__ __forceinline__ void read_all(uint32_t tile, const Addr &ad)
     {
@@ -454,6 +464,7 @@ gemm_x16_kernel(const GemmArgs args)
         uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, lbuf), dst_b = op_dst(std::integral_constant<int, 1>{}, lbuf);
         if constexpr (load_mode != 0 && PAIR) asm volatile("" : "+s"(dst_x0), "+s"(dst_x1));
         if constexpr (load_mode != 0 && !PAIR) asm volatile("" : "+s"(dst_a), "+s"(dst_b));
+        uint32_t read_a[FragA::NADDR], read_b[FragB::NADDR];      // addresses of the LDS reads, each live from its first use to its last
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
             // boustrophedon over the FM x FN blocks: consecutive MFMAs share one operand register, also at the row
@@ -478,16 +489,29 @@ gemm_x16_kernel(const GemmArgs args)
                 else if constexpr (l0 < TileA::LPW) set_lds_destination(dst_a + l0 * 1024);
                 else set_lds_destination(dst_b + (l0 - TileA::LPW) * 1024);
             }
+            // An address that a read of this slot is the first to use is worked out BEFORE the MFMA (the empty asm, which only
+            // reads it, keeps the addition there): behind it, the read would wait for the addition with nothing in between,
+            // and where the compiler puts it otherwise changes with unrelated code (measured: 2-3 % at 8192^3 fp16 NN).
+            constexpr int r0 = m < READ_SPAN ? NR * m / READ_SPAN : 0, r1 = m < READ_SPAN ? NR * (m + 1) / READ_SPAN : 0;
+            static_for<r1 - r0>([&](auto RR) {
+                constexpr int r = r0 + decltype(RR)::value;
+                if constexpr (r < NA) {
+                    if constexpr (FragA::first_use(r)) {
+                        read_a[FragA::address_index(r)] = t + adA.a[FragA::address_index(r)];
+                        asm volatile("" ::"v"(read_a[FragA::address_index(r)]));
+                    }
+                } else if constexpr (FragB::first_use(r - NA)) {
+                    read_b[FragB::address_index(r - NA)] = t + TileA::BYTES + adB.a[FragB::address_index(r - NA)];
+                    asm volatile("" ::"v"(read_b[FragB::address_index(r - NA)]));
+                }
+            });
             if constexpr (ESZ == 2) mfma_acc<(i * FN + j) * 4, NACC>(ca.x[i], cb.x[j]);
             else mfma_acc_f32<(i * FN + j) * 4, NACC>(ca.x[i][tt], cb.x[j][tt]);
-            if constexpr (m < READ_SPAN) {
-                constexpr int r0 = NR * m / READ_SPAN, r1 = NR * (m + 1) / READ_SPAN;
-                static_for<r1 - r0>([&](auto RR) {
-                    constexpr int r = r0 + decltype(RR)::value;
-                    if constexpr (r < NA) na.template read_op<r>(t, adA);
-                    else nb.template read_op<r - NA>(t + TileA::BYTES, adB);
-                });
-            }
+            static_for<r1 - r0>([&](auto RR) {
+                constexpr int r = r0 + decltype(RR)::value;
+                if constexpr (r < NA) na.template read_op_at<r>(read_a[FragA::address_index(r)]);
+                else nb.template read_op_at<r - NA>(read_b[FragB::address_index(r - NA)]);
+            });
             constexpr std::bool_constant<single> DESTINATION_SET{};
             static_for<n_second>([&](auto LL) {
                 constexpr int l = p0 + decltype(LL)::value;
@@ -797,19 +821,33 @@ gemm_x16_kernel(const GemmArgs args)
         // of the lower block, so every lane stores 16 contiguous bytes and a column gets 64 per instruction.
         const uint32_t q = lane >> 4;
         const uint32_t prow0 = row0 + wm * Cfg::TM + ((q & 1) ? 4 * q + 12 : 4 * q);
-        static_for<FM * FN / 2>([&](auto IJ) {
-            constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
-            constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
-            union { T e[4]; uint32_t u[2]; } x, y;
-            x.e[0] = (T)(alpha * acc_read<b0>());     x.e[1] = (T)(alpha * acc_read<b0 + 1>());
-            x.e[2] = (T)(alpha * acc_read<b0 + 2>()); x.e[3] = (T)(alpha * acc_read<b0 + 3>());
-            y.e[0] = (T)(alpha * acc_read<b1>());     y.e[1] = (T)(alpha * acc_read<b1 + 1>());
-            y.e[2] = (T)(alpha * acc_read<b1 + 2>()); y.e[3] = (T)(alpha * acc_read<b1 + 3>());
-            auto s0 = __builtin_amdgcn_permlane16_swap(x.u[0], y.u[0], false, false);
-            auto s1 = __builtin_amdgcn_permlane16_swap(x.u[1], y.u[1], false, false);
-            T *p = C + (size_t)(wcol0 + j * 16) * ldc + prow0 + i * 16;
-            *reinterpret_cast<u32x4 *>(p) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
-        });
+        // Two results at a time go through the packed conversion (round to nearest even, like the scalar cast), and
+        // alpha == 1 gets a copy of the sequence without the multiplications: 4 (12) instructions per eight results where
+        // scalar casts took 16.  The epilogue is bound by instruction issue, and a resident work-group pays it per tile.
+        auto two = [](float a, float b) -> uint32_t {
+            typedef float f32x2 __attribute__((ext_vector_type(2)));
+            typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+            return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
+        };
+        auto store_all = [&](auto UNIT_ALPHA) {
+            constexpr bool unit = decltype(UNIT_ALPHA)::value;
+            static_for<FM * FN / 2>([&](auto IJ) {
+                constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
+                constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
+                float x[4] = {acc_read<b0>(), acc_read<b0 + 1>(), acc_read<b0 + 2>(), acc_read<b0 + 3>()};
+                float y[4] = {acc_read<b1>(), acc_read<b1 + 1>(), acc_read<b1 + 2>(), acc_read<b1 + 3>()};
+                if constexpr (!unit) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) { x[r] *= alpha; y[r] *= alpha; }
+                }
+                auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
+                auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
+                T *p = C + (size_t)(wcol0 + j * 16) * ldc + prow0 + i * 16;
+                *reinterpret_cast<u32x4 *>(p) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
+            });
+        };
+        if (alpha == 1.0f) store_all(std::true_type{});
+        else store_all(std::false_type{});
     } else if (vec_c) {
         static_for<FM * FN>([&](auto IJ) {
             constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
