@@ -33,26 +33,6 @@ using ring::slice_cursor;
 using ring::static_for;
 using ring::uniform_address;
 
-#define MMBO_AGPR_0_63 \
-    "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15" , \
-    "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31" , \
-    "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47" , \
-    "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63"
-#define MMBO_AGPR_64_127 \
-    "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79" , \
-    "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95" , \
-    "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111" , \
-    "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127"
-#define MMBO_AGPR_128_255 \
-    "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143" , \
-    "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159" , \
-    "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175" , \
-    "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191" , \
-    "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207" , \
-    "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223" , \
-    "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239" , \
-    "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
-
 // The 64 accumulator blocks a[4q : 4q+3], spelled out: an asm statement names its registers and its clobbers as literals.
 #define MMBO_ACC_BLOCKS(X) \
     X(0,1,2,3) X(4,5,6,7) X(8,9,10,11) X(12,13,14,15) X(16,17,18,19) X(20,21,22,23) X(24,25,26,27) X(28,29,30,31) \
@@ -93,17 +73,18 @@ __device__ __forceinline__ void mfma_acc_f32(uint32_t a, uint32_t b)
     MMBO_ACC_BLOCKS(X)
 #undef X
 }
+// All NACC accumulation registers = 0, four per statement, each statement clobbering the four it writes (between
+// statements that each name every register the compiler would put one s_nop per write); together the statements name
+// all of them, which is what keeps the compiler from using any.
 template <int NACC>
 __device__ __forceinline__ void acc_zero()
 {
-    static_for<NACC>([&](auto I) {
-        if constexpr (NACC > 128)
-            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63, MMBO_AGPR_64_127, MMBO_AGPR_128_255);
-        else if constexpr (NACC > 64)
-            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63, MMBO_AGPR_64_127);
-        else
-            asm volatile("v_accvgpr_write_b32 a[%0], 0" :: "n"(decltype(I)::value) : MMBO_AGPR_0_63);
-    });
+#define X(r0, r1, r2, r3)                                                                                              \
+    if constexpr (r0 < NACC)                                                                                           \
+        asm volatile("v_accvgpr_write_b32 a[" #r0 "], 0\n\tv_accvgpr_write_b32 a[" #r1 "], 0\n\t"                      \
+                     "v_accvgpr_write_b32 a[" #r2 "], 0\n\tv_accvgpr_write_b32 a[" #r3 "], 0" ::: "a" #r0, "a" #r1, "a" #r2, "a" #r3);
+    MMBO_ACC_BLOCKS(X)
+#undef X
     asm volatile("s_nop 7" ::: "memory");
 }
 template <int I>
@@ -430,7 +411,6 @@ gemm_x16_kernel(const GemmArgs args)
     const typename FragB::Addr adB = FragB::make_addr(lane, wn * Cfg::TN);
     FragA fa[2];
     FragB fb[2];
-    acc_zero<NACC>();
 
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
@@ -557,6 +537,7 @@ gemm_x16_kernel(const GemmArgs args)
 #pragma unroll
         for (int q = 0; q < DEPTH; ++q)
             if (q < n_slice) issue_slice(q);
+        acc_zero<NACC>();                                                // (while the first slices are on their way)
         if (n_slice >= DEPTH) MMBO_WAIT_VM(BATCH * (DEPTH - 1)); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slice 0 resident
         read_slice(fa[0], fb[0], 0);
@@ -611,6 +592,7 @@ gemm_x16_kernel(const GemmArgs args)
             }
         }
         constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
+        acc_zero<NACC>();                                                // (while the first slices are on their way)
         if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - BATCH); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slice 0 resident
         read_slice(fa[0], fb[0], 0);
@@ -786,7 +768,50 @@ gemm_x16_kernel(const GemmArgs args)
     T *C = static_cast<T *>(args.C) + (int64_t)batch * args.strideC;
     const bool vec_c = args.vec_c != 0;
     typedef typename std::conditional<ESZ == 2, u32x2, u32x4>::type cvec;       // four consecutive rows of one column
+    // fp16: a lane's four rows are 8 bytes, a column of one block 32 bytes -- a quarter of a cache line per request.  Two
+    // vertically adjacent blocks therefore travel together: v_permlane16_swap hands the lanes of the even 16-lane rows their
+    // lower neighbour's four rows of the upper block and the odd rows their upper neighbour's of the lower block, so every
+    // lane stores 16 contiguous bytes, from row pair_row0 of the pair on, and a column gets 64 per instruction.  The
+    // exchange is its own inverse: applied to a vector loaded from there it returns each lane its rows of both blocks.
+    // Two results at a time go through the packed conversion (round to nearest even, like the scalar cast).
+    constexpr bool PAIRED_C = ESZ == 2 && FM % 2 == 0;
+    const uint32_t pair_row0 = row0 + wm * Cfg::TM + (((lane >> 4) & 1) ? 4 * (lane >> 4) + 12 : 4 * (lane >> 4));
+    auto two = [](float a, float b) -> uint32_t {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
+    };
     if (vec_c && beta != 0.0f) {
+        if constexpr (PAIRED_C) {
+            // the whole wave tile of old C is requested before its first value is used (see below)
+            u32x4 cold[FM * FN / 2];
+            static_for<FM * FN / 2>([&](auto IJ) {
+                constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
+                cold[decltype(IJ)::value] = *reinterpret_cast<const u32x4 *>(C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16);
+            });
+            static_for<FM * FN / 2>([&](auto IJ) {
+                constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
+                constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
+                const u32x4 c = cold[decltype(IJ)::value];
+                auto o0 = __builtin_amdgcn_permlane16_swap(c[0], c[2], false, false);
+                auto o1 = __builtin_amdgcn_permlane16_swap(c[1], c[3], false, false);
+                union { T e[4]; uint32_t u[2]; } xo, yo;
+                xo.u[0] = o0[0]; xo.u[1] = o1[0];
+                yo.u[0] = o0[1]; yo.u[1] = o1[1];
+                float x[4] = {alpha * acc_read<b0>(), alpha * acc_read<b0 + 1>(), alpha * acc_read<b0 + 2>(), alpha * acc_read<b0 + 3>()};
+                float y[4] = {alpha * acc_read<b1>(), alpha * acc_read<b1 + 1>(), alpha * acc_read<b1 + 2>(), alpha * acc_read<b1 + 3>()};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    x[r] = __builtin_fmaf(beta, (float)xo.e[r], x[r]);
+                    y[r] = __builtin_fmaf(beta, (float)yo.e[r], y[r]);
+                }
+                auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
+                auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
+                T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
+                *reinterpret_cast<u32x4 *>(p) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
+            });
+            continue;
+        }
         // beta != 0 (reference: the fma(C, beta, .) epilogue, MT192x096x08 kernel :3037-3056): a whole column strip of
         // old C (fp16: the whole wave tile) is requested before its first value is used, so the read-modify-write runs
         // at memory bandwidth instead of one load latency per block.
@@ -814,21 +839,9 @@ gemm_x16_kernel(const GemmArgs args)
     // beta == 0: C is never read.  The aligned and the element-wise variant are separate straight-line sequences: with
     // the choice made per block the epilogue was bound by instruction issue (64 blocks x ~20 instructions with two
     // branches each took 7 us of a 220 us tile at 8192^3, whatever the number of work-groups writing at the time).
-    if (vec_c && ESZ == 2 && FM % 2 == 0) {
-        // fp16: a lane's four rows are 8 bytes, a column of one block 32 bytes -- a quarter of a cache line per write
-        // request.  Two vertically adjacent blocks are stored together: v_permlane16_swap hands the lanes of the even
-        // 16-lane rows their lower neighbour's four rows of the upper block and the odd rows their upper neighbour's
-        // of the lower block, so every lane stores 16 contiguous bytes and a column gets 64 per instruction.
-        const uint32_t q = lane >> 4;
-        const uint32_t prow0 = row0 + wm * Cfg::TM + ((q & 1) ? 4 * q + 12 : 4 * q);
-        // Two results at a time go through the packed conversion (round to nearest even, like the scalar cast), and
-        // alpha == 1 gets a copy of the sequence without the multiplications: 4 (12) instructions per eight results where
-        // scalar casts took 16.  The epilogue is bound by instruction issue, and a resident work-group pays it per tile.
-        auto two = [](float a, float b) -> uint32_t {
-            typedef float f32x2 __attribute__((ext_vector_type(2)));
-            typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-            return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2{a, b}), f16x2));
-        };
+    if (vec_c && PAIRED_C) {
+        // alpha == 1 gets a copy of the sequence without the multiplications: with the packed conversions that makes 4 (12)
+        // instructions per eight results where scalar casts took 16.
         auto store_all = [&](auto UNIT_ALPHA) {
             constexpr bool unit = decltype(UNIT_ALPHA)::value;
             static_for<FM * FN / 2>([&](auto IJ) {
@@ -842,7 +855,7 @@ gemm_x16_kernel(const GemmArgs args)
                 }
                 auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
                 auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
-                T *p = C + (size_t)(wcol0 + j * 16) * ldc + prow0 + i * 16;
+                T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
                 *reinterpret_cast<u32x4 *>(p) = u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]};
             });
         };
