@@ -290,6 +290,28 @@ def test_x16_kernel_chip_block_order_and_refusals():
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+@pytest.mark.parametrize("ta", [0, 1])
+@pytest.mark.parametrize("tb", [0, 1])
+def test_x16_resident_work_groups_walk_several_tiles(dtype, ta, tb):
+    """More 256 x 256 tiles than CUs: a work-group stays resident and takes several tiles, one after the other through
+    the same ring -- whole tiles with even and odd slice counts, a partial last slice, a ragged last tile row -- against
+    the oracle, with beta = 0 over NaN-filled C and with a read-modify-write, and in a batch of two problems."""
+    cid = _x16_ids(dtype)[0]
+    slice_k = 32 if dtype == F16 else 16
+    dist = "normal" if dtype == F16 else "uniform"
+    cases = [(4352, 4352, 10 * slice_k, 1, 0.0),          # 289 tiles, twice the ring depth in slices
+             (4352, 4608, 22 * slice_k, 1, 0.5),          # C read and written
+             (4608, 4352, 11 * slice_k, 1, 0.0),          # odd slice count
+             (4352, 4352, 12 * slice_k + 5, 1, 0.0),      # partial last slice
+             (4352 - 8, 4352, 12 * slice_k, 1, 0.0),      # ragged last tile row
+             (4352, 4352, 12 * slice_k, 2, 1.0)]          # two problems, 289 tiles each
+    for (m, n, k, batch, beta) in cases:
+        p = U.Problem(dtype, ta, tb, m, n, k, 1.25, beta, batch=batch, seed=900 + k + batch, dist=dist,
+                      c_fill="uniform" if beta else "nan")
+        _run_and_check(p, cid, label=f"resident {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch} beta={beta}")
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_ring_kernel_refuses_shapes_it_cannot_take(dtype):
     """Ragged m/n, k that does not split into whole slices, unaligned A: MMBO_ERR_INVALID_CONFIG, never a wrong
     result; the automatic pick moves to a kernel that takes the problem and still matches the oracle."""
