@@ -47,7 +47,7 @@ def profiled_traffic(head, tile_config):
     return float(m.group(1)) + float(m.group(2)), f"{TRAFFIC_PROFILE[head]} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, taken {m.group(4)})"
 
 
-def timed_launches(torch, stream, step, steps, warmup, settle=True, groups=None):
+def timed_launches(torch, stream, step, steps, warmup, settle=True, groups=None, settle_min_ms=100.0, settle_max_ms=600.0):
     """warm-up, settle phase, then exactly `steps` launches in event-delimited groups (one per launch up to 25 groups).
     Returns a dict: median/mean/min/max per-launch ms over the groups, wall ms per launch, settle figures."""
     for _ in range(warmup):
@@ -55,7 +55,8 @@ def timed_launches(torch, stream, step, steps, warmup, settle=True, groups=None)
     torch.cuda.synchronize()
     settle_ms, settle_n = 0.0, 0
     if settle:
-        # launch in chunks until >= 100 ms have passed and two consecutive chunks agree within 1.5 % (at most 600 ms)
+        # launch in chunks until >= settle_min_ms (100 ms) have passed and two consecutive chunks agree within 1.5 %
+        # (at most settle_max_ms, 600 ms)
         t_begin = time.perf_counter()
         prev = None
         chunk = 4
@@ -70,7 +71,7 @@ def timed_launches(torch, stream, step, steps, warmup, settle=True, groups=None)
             settle_n += chunk
             settle_ms = (time.perf_counter() - t_begin) * 1e3
             stable = prev is not None and abs(cur - prev) <= 0.015 * prev
-            if (settle_ms >= 100.0 and stable) or settle_ms >= 600.0:
+            if (settle_ms >= settle_min_ms and stable) or settle_ms >= settle_max_ms:
                 break
             prev = cur
             if cur * chunk < 10.0:
@@ -195,7 +196,7 @@ def skinny_legs(G, torch, steps, warmup):
             cid = G.select_config(dtype, 0, 0, m, n, k, 1)
             # small kernels: ten groups of at least twenty back-to-back launches each, median over the groups
             us = timed_launches(torch, stream, lambda: G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream),
-                                max(steps, 200), max(warmup, 20), settle=False, groups=10)["median_ms"] * 1e3
+                                max(steps, 200), max(warmup, 20), groups=10, settle_min_ms=30.0, settle_max_ms=200.0)["median_ms"] * 1e3
             nbytes = (m * k + k * n + m * n) * esz
             out[f"{dname}_{m}x{n}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / us * 1e-3, 1),
                                             "frac_of_hbm_peak": round(nbytes / us * 1e-3 / 8000.0, 4),
@@ -223,7 +224,7 @@ def ragged_legs(G, torch, steps, warmup):
 
         def run():
             G.gemm(dtype, ta, tb, m, n, k, 1.0, A, lda, B, ldb, 0.0, C, m, G.CONFIG_AUTO, stream)
-        us = timed_launches(torch, stream, run, max(steps, 20), max(warmup, 5), settle=False, groups=10)["median_ms"] * 1e3
+        us = timed_launches(torch, stream, run, max(steps, 20), max(warmup, 5), groups=10, settle_min_ms=30.0, settle_max_ms=200.0)["median_ms"] * 1e3
         tf = 2.0 * m * n * k / us * 1e-6
         out[f"{dname}_{'NT'[ta]}{'NT'[tb]}_{m}x{n}x{k}"] = {"us": round(us, 1), "tflops": round(tf, 1),
                                                             "frac_of_peak": round(tf / PEAK_TFLOPS["f16" if dtype == G.F16 else "f32"], 4),
@@ -257,7 +258,7 @@ def config_legs(G, torch, steps, warmup):
             G.gemm_strided_batched(dtype, ta, tb, m, n, k, alpha, A, lda, m * k, B, ldb, k * n, beta, C, m, m * n, batch,
                                    G.CONFIG_AUTO, stream)
         reps = max(steps, 20) if m >= 4096 else max(steps, 200)
-        us = timed_launches(torch, stream, run, reps, max(warmup, 10), settle=False, groups=10)["median_ms"] * 1e3
+        us = timed_launches(torch, stream, run, reps, max(warmup, 10), groups=10, settle_min_ms=30.0, settle_max_ms=200.0)["median_ms"] * 1e3
         tf = 2.0 * m * n * k * batch / us * 1e-6
         esz = 2 if dtype == G.F16 else 4
         gbps = batch * (m * k + k * n + m * n * (2 if beta != 0 else 1)) * esz / us * 1e-3
