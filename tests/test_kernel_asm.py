@@ -256,6 +256,10 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
                                          "v_accvgpr_read_b32")), (name, t)
                     if t.startswith("v_accvgpr_write_b32"):
                         assert re.match(r"v_accvgpr_write_b32 a\[?\w+\]?, 0$", t), (name, t)
+            # and none of that is the compiler's own: every instruction that names an accumulation register sits inside an asm
+            # statement (under register pressure the compiler parks values of its own in accumulation registers)
+            own = [t for t in _compiler_generated(path)[name] if re.search(r"\ba\[?\d", t)]
+            assert not own, (name, own[:3])
             m = re.search(r"\.amdhsa_kernel " + re.escape(name) + r"\b.*?\.amdhsa_next_free_vgpr (\d+).*?\.amdhsa_accum_offset (\d+)",
                           text, re.S)
             assert m, name
