@@ -153,7 +153,7 @@ def dgemm_legs(G, torch, steps, warmup):
         C0 = torch.rand(m * n, device="cuda", generator=gen, dtype=torch.float64)
         C = C0.clone()
         cid = G.select_config(G.F64, ta, tb, m, n, k, 1)
-        nsteps = max(3, steps // 5) if tag == "8192" else steps
+        nsteps = max(10, steps // 2) if tag == "8192" else max(10, steps)
         ms = timed_launches(torch, stream, lambda: G.gemm(G.F64, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, m, cid, stream),
                             nsteps, max(2, warmup // 4), settle=False)["median_ms"]
         # parity on a band of 64 rows of one fresh application (beta = 1 accumulates over the timed launches)
@@ -311,7 +311,8 @@ def main():
     for name, dtype in (("f16", G.F16), ("f32", G.F32)):
         if args.only and args.only != name:
             continue
-        steps = args.steps if name == "f16" else max(3, args.steps // 5)
+        # (the fp32 launch takes ten times as long: half the launches, but never fewer than ten timed groups)
+        steps = args.steps if name == "f16" else max(10, args.steps // 2)
         warm = args.warmup if name == "f16" else max(2, args.warmup // 5)
         t, cfg, tensors = time_gemm(G, torch, dtype, m, n, k, steps, warm, seed=1234)
         rel, limit, host = spot_check(G, dtype, m, n, k, *tensors)
@@ -345,8 +346,8 @@ def main():
         print(json.dumps({"metric": METRIC, "also": f64}))
         return
     ceilings = {}
-    if not args.only:
-        for name, dtype in (("f16", G.F16), ("f32", G.F32), ("f64", G.F64)):
+    for name, dtype in (("f16", G.F16), ("f32", G.F32), ("f64", G.F64)):
+        if not args.only or args.only == name:          # (a one-leg run, as the profiles use, probes that leg's type only)
             for rnd in (0, 1):
                 tf, mhz = G.probe_mfma_ceiling(dtype, bool(rnd))
                 ceilings[f"{name}_{'random' if rnd else 'ones'}_operands"] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
@@ -390,6 +391,7 @@ def main():
         out["also"] = {"fp32_tflops": round(flops / q["ev_ms"] * 1e-9, 2), "fp32_ms_per_step": round(q["ev_ms"], 4),
                        "fp32_frac_of_peak": round(flops / q["ev_ms"] * 1e-9 / PEAK_TFLOPS["f32"], 4),
                        "fp32_peak": PEAK_TFLOPS["f32"], "fp32_tile_config": q["cfg"]["name"], "fp32_steps": q["steps"],
+                       "fp32_groups": q["t"]["groups"],
                        "fp32_max_rel_err": float(f"{q['rel']:.3e}"), "fp32_rel_err_limit": float(f"{q['limit']:.3e}")}
     if ones_tflops is not None:
         out.setdefault("also", {})["fp16_constant_operands_tflops"] = round(ones_tflops, 1)

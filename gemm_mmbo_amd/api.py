@@ -20,7 +20,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmmbo_gemm.so")
 EXPORTS = (
     "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_gemm_strided_batched_static_workspace", "mmbo_static_workspace_bytes",
     "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
-    "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_batch_xcd_remap", "mmbo_release_workspace", "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
+    "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_batch_xcd_remap", "mmbo_release_workspace", "mmbo_release_stream_workspace", "mmbo_workspace_info",
+    "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
 
@@ -74,6 +75,10 @@ def lib():
         L.mmbo_batch_xcd_remap.argtypes = [cu, cu, cu, ctypes.POINTER(cu), ctypes.POINTER(cu)]
         L.mmbo_batch_xcd_remap.restype = ci
         L.mmbo_release_workspace.restype = ci
+        L.mmbo_release_stream_workspace.argtypes = [vp]
+        L.mmbo_release_stream_workspace.restype = ci
+        L.mmbo_workspace_info.argtypes = [ctypes.POINTER(sz), ctypes.POINTER(sz)]
+        L.mmbo_workspace_info.restype = ci
         dp = ctypes.POINTER(ctypes.c_double)
         L.mmbo_probe_mfma_ceiling.argtypes = [ci, ci, dp, dp]
         L.mmbo_probe_mfma_ceiling.restype = ci
@@ -195,6 +200,18 @@ def probe_mfma_ceiling(dtype, random_operands=True):
 
 def release_workspace():
     _check(lib().mmbo_release_workspace())
+
+
+def release_stream_workspace(stream):
+    """Frees the split-K workspace the library holds for `stream` (waits for that stream only)."""
+    _check(lib().mmbo_release_stream_workspace(_stream_handle(stream)))
+
+
+def workspace_info():
+    """(number of split-K workspaces held for the current device, their total bytes)."""
+    slots, nbytes = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    _check(lib().mmbo_workspace_info(ctypes.byref(slots), ctypes.byref(nbytes)))
+    return slots.value, nbytes.value
 
 
 def version():

@@ -29,6 +29,36 @@ FLAGS = [
 ]
 
 
+# The direct-to-LDS kernels rely on facts about the generated code that the compiler does not guarantee: their inline
+# assembly changes M0 and the accumulation registers without declaring it, and LDS reads stay in flight across
+# compiler-scheduled instructions.  tests/test_kernel_asm.py checks those facts on the assembly a given hipcc generates;
+# this is the compiler build it last passed with.  Another compiler may still be fine -- run that test file with it
+# first (then update this string); MMBO_STRICT_TOOLCHAIN=1 turns the warning below into an error.
+ASM_CHECKED_WITH = "roc-7.2.0 26014"
+
+
+def _hipcc_version():
+    try:
+        return subprocess.run([HIPCC, "--version"], capture_output=True, text=True).stdout
+    except OSError as e:
+        raise RuntimeError(f"cannot run {HIPCC}: {e}")
+
+
+def _check_toolchain(verbose=True):
+    text = _hipcc_version()
+    if ASM_CHECKED_WITH in text:
+        return True
+    first = (text.strip().split("\n") or ["?"])[0:2]
+    msg = (f"gemm_mmbo_amd.build: {HIPCC} is not the compiler build the kernels' assembly checks passed with "
+           f"(want '{ASM_CHECKED_WITH}', have: {' / '.join(first)}).  Run `python -m pytest tests/test_kernel_asm.py` with this "
+           "compiler before trusting the library.")
+    if os.environ.get("MMBO_STRICT_TOOLCHAIN") == "1":
+        raise RuntimeError(msg)
+    if verbose:
+        print("WARNING: " + msg, file=sys.stderr)
+    return False
+
+
 def _units():
     units = [("mmbo_gemm.hip", "mmbo_gemm.o", []), ("probe.hip", "probe.o", [])]
     for dtype in (0, 1):
@@ -43,12 +73,6 @@ def _units():
             units.append(("inst_x16.hip", f"inst_x16_{dtype}_{tile}.o", [f"-DMMBO_DTYPE={dtype}", f"-DMMBO_TILE={tile}"]))
     for tile in range(NUM_F64_TILES):
         units.append(("inst_dgemm.hip", f"inst_dgemm_{tile}.o", [f"-DMMBO_TILE={tile}"]))
-    extra = os.path.join(CSRC, "extra_units.txt")
-    if os.path.exists(extra):
-        for line in open(extra):
-            line = line.split("#")[0].split()
-            if line:
-                units.append((line[0], line[1], line[2:]))
     return units
 
 
@@ -80,8 +104,8 @@ def _compile(unit, force, newest_dep):
 
 def build(force=False, verbose=True, jobs=None):
     os.makedirs(OBJ, exist_ok=True)
-    extra = os.path.join(CSRC, "extra_units.txt")
-    newest = max(os.path.getmtime(p) for p in (os.path.abspath(__file__), extra) if os.path.exists(p))
+    _check_toolchain(verbose)
+    newest = os.path.getmtime(os.path.abspath(__file__))
     units = _units()
     jobs = jobs or min(8, os.cpu_count() or 1)
     with ThreadPoolExecutor(max_workers=jobs) as ex:

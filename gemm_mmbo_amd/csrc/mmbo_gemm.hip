@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -68,57 +69,157 @@ int hip_fail(hipError_t e)
 constexpr int kMaxDevices = 64;
 
 // Library-owned workspaces: one per (device, stream), so GEMMs on different streams never share partial sums, grown on
-// demand.  Only launches on that stream ever touch a slot's buffer, so growing it waits for that stream alone.  The
-// mutex is held from the lookup until the launches that use the buffer have been queued: another host thread that
-// grows (frees) the same stream's buffer then does so after them in stream order.
+// demand, at most kMaxWsSlots per device (the reference's launcher never frees what it loads, src/gemm/driver.h:41; this
+// table is bounded instead).
+//   - Each device has its own table and table lock, held only to look a slot up, add one or take one out.
+//   - Each slot has its own lock, held by a call from the lookup until both launches that use the buffer (the GEMM and
+//     the reduction) are queued: two host threads on one stream cannot interleave their launches, and growing a buffer
+//     (wait for that stream, free, allocate) stalls only callers of that same stream.
+//   - A new stream that finds the table full retires the least recently used slot nobody holds: the table lock is given
+//     up, the device is synchronised (the slot's stream may no longer exist, so it cannot be waited for by handle) and
+//     the buffer freed.  mmbo_release_stream_workspace retires one stream's slot at the caller's request.
+constexpr size_t kMaxWsSlots = 8;
 struct WsSlot {
-    hipStream_t stream;
-    char *base;
-    size_t bytes;
+    hipStream_t stream = nullptr;
+    char *base = nullptr;
+    size_t bytes = 0;
+    unsigned long long last_use = 0;
+    bool dead = false;          // taken out of the table; whoever still holds a reference looks the stream up again
+    std::mutex use;
 };
-std::mutex g_ws_mutex;
-std::vector<WsSlot> g_ws_slots[kMaxDevices];
+struct WsTable {
+    std::mutex lock;
+    std::vector<std::shared_ptr<WsSlot>> slots;
+    unsigned long long clock = 0;
+};
+WsTable g_ws[kMaxDevices];
 
-// The buffer of (current device, stream), at least `bytes` large.  Caller holds g_ws_mutex.
-int workspace(hipStream_t stream, size_t bytes, char **out)
+// A held slot: its buffer may be used until the holder is destroyed.
+struct WsHold {
+    std::shared_ptr<WsSlot> slot;
+    std::unique_lock<std::mutex> held;
+};
+
+// The buffer of (current device, stream), at least `bytes` large, held for the caller.
+int workspace(hipStream_t stream, size_t bytes, WsHold &hold, char **out)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e);
     if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
-    std::vector<WsSlot> &slots = g_ws_slots[dev];
-    WsSlot *slot = nullptr;
-    for (WsSlot &sl : slots)
-        if (sl.stream == stream) slot = &sl;
-    if (!slot) {
-        slots.push_back(WsSlot{stream, nullptr, 0});
-        slot = &slots.back();
-    }
-    if (slot->bytes < bytes) {
-        if (slot->base) {
-            // earlier launches on this stream may still be using the old buffer (fails under stream capture: a captured
-            // call must find its workspace already large enough, or use the entry point that allocates nothing)
-            e = hipStreamSynchronize(stream);
-            if (e != hipSuccess) return hip_fail(e);
-            (void)hipFree(slot->base);
-            slot->base = nullptr;
-            slot->bytes = 0;
+    WsTable &tab = g_ws[dev];
+    for (;;) {
+        std::shared_ptr<WsSlot> slot, victim;
+        std::unique_lock<std::mutex> victim_held;
+        {
+            std::lock_guard<std::mutex> tl(tab.lock);
+            for (auto &sl : tab.slots)
+                if (sl->stream == stream) slot = sl;
+            if (!slot) {
+                if (tab.slots.size() >= kMaxWsSlots) {
+                    // retire the least recently used slot that no call holds
+                    size_t pick = tab.slots.size();
+                    for (size_t i = 0; i < tab.slots.size(); ++i) {
+                        if (pick < tab.slots.size() && tab.slots[i]->last_use >= tab.slots[pick]->last_use) continue;
+                        std::unique_lock<std::mutex> t(tab.slots[i]->use, std::try_to_lock);
+                        if (!t.owns_lock()) continue;
+                        pick = i;
+                        victim_held = std::move(t);
+                    }
+                    if (pick < tab.slots.size()) {
+                        victim = tab.slots[pick];
+                        victim->dead = true;
+                        tab.slots.erase(tab.slots.begin() + (long)pick);
+                    }
+                    // (every slot held by a call in flight: the table grows past its bound for now)
+                }
+                slot = std::make_shared<WsSlot>();
+                slot->stream = stream;
+                tab.slots.push_back(slot);
+            }
+            slot->last_use = ++tab.clock;
         }
-        size_t want = bytes + bytes / 4;
-        void *p = nullptr;
-        if (hipMalloc(&p, want) != hipSuccess) {
-            (void)hipGetLastError();
-            want = bytes;
+        if (victim) {
+            if (victim->base) {
+                e = hipDeviceSynchronize();
+                (void)hipFree(victim->base);
+                victim->base = nullptr;
+                victim->bytes = 0;
+            }
+            victim_held.unlock();
+            if (e != hipSuccess) return hip_fail(e);
+        }
+        std::unique_lock<std::mutex> held(slot->use);
+        if (slot->dead) continue;                    // retired between the lookup and here: look the stream up again
+        if (slot->bytes < bytes) {
+            if (slot->base) {
+                // earlier launches on this stream may still be using the old buffer (fails under stream capture: a captured
+                // call must find its workspace already large enough, or use the entry point that allocates nothing)
+                e = hipStreamSynchronize(stream);
+                if (e != hipSuccess) return hip_fail(e);
+                (void)hipFree(slot->base);
+                slot->base = nullptr;
+                slot->bytes = 0;
+            }
+            size_t want = bytes + bytes / 4;
+            void *p = nullptr;
             if (hipMalloc(&p, want) != hipSuccess) {
                 (void)hipGetLastError();
-                return MMBO_ERR_WORKSPACE;
+                want = bytes;
+                if (hipMalloc(&p, want) != hipSuccess) {
+                    (void)hipGetLastError();
+                    return MMBO_ERR_WORKSPACE;
+                }
+            }
+            slot->base = static_cast<char *>(p);
+            slot->bytes = want;
+        }
+        *out = slot->base;
+        hold.slot = std::move(slot);
+        hold.held = std::move(held);
+        return MMBO_OK;
+    }
+}
+
+// Takes the slots `which` selects out of the current device's table and frees their buffers.  `stream_only`: wait for
+// that stream alone (its handle is still valid: the caller is about to destroy it); otherwise for the whole device.
+int release_slots(bool stream_only, hipStream_t stream)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e);
+    if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
+    WsTable &tab = g_ws[dev];
+    std::vector<std::shared_ptr<WsSlot>> out;
+    {
+        std::lock_guard<std::mutex> tl(tab.lock);
+        for (size_t i = 0; i < tab.slots.size();) {
+            if (!stream_only || tab.slots[i]->stream == stream) {
+                out.push_back(tab.slots[i]);
+                tab.slots.erase(tab.slots.begin() + (long)i);
+            } else {
+                ++i;
             }
         }
-        slot->base = static_cast<char *>(p);
-        slot->bytes = want;
     }
-    *out = slot->base;
-    return MMBO_OK;
+    if (out.empty()) return MMBO_OK;
+    hipError_t first = hipSuccess;
+    for (auto &sl : out) {
+        std::lock_guard<std::mutex> held(sl->use);       // a call that holds the slot queues its launches first
+        sl->dead = true;
+    }
+    e = stream_only ? hipStreamSynchronize(stream) : hipDeviceSynchronize();
+    if (e != hipSuccess) return hip_fail(e);
+    for (auto &sl : out) {
+        std::lock_guard<std::mutex> held(sl->use);
+        if (sl->base) {
+            e = hipFree(sl->base);
+            if (e != hipSuccess && first == hipSuccess) first = e;
+            sl->base = nullptr;
+            sl->bytes = 0;
+        }
+    }
+    return first == hipSuccess ? MMBO_OK : hip_fail(first);
 }
 
 // The workspace of the entry point that allocates nothing: one array per device in the library's own image, there from
@@ -529,25 +630,22 @@ int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, uns
     return MMBO_OK;
 }
 
-int mmbo_release_workspace(void)
+int mmbo_release_workspace(void) { return release_slots(false, nullptr); }
+
+int mmbo_release_stream_workspace(void *stream) { return release_slots(true, static_cast<hipStream_t>(stream)); }
+
+int mmbo_workspace_info(size_t *slots, size_t *bytes)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e);
     if (dev < 0 || dev >= kMaxDevices) return MMBO_ERR_NO_DEVICE;
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (!g_ws_slots[dev].empty()) {
-        e = hipDeviceSynchronize();
-        if (e != hipSuccess) return hip_fail(e);
-        hipError_t first = hipSuccess;
-        for (WsSlot &sl : g_ws_slots[dev])
-            if (sl.base) {
-                e = hipFree(sl.base);
-                if (e != hipSuccess && first == hipSuccess) first = e;
-            }
-        g_ws_slots[dev].clear();
-        if (first != hipSuccess) return hip_fail(first);
-    }
+    WsTable &tab = g_ws[dev];
+    std::lock_guard<std::mutex> tl(tab.lock);
+    size_t total = 0;
+    for (auto &sl : tab.slots) total += sl->bytes;          // (a size being changed right now may be read stale: a diagnostic)
+    if (slots) *slots = tab.slots.size();
+    if (bytes) *bytes = total;
     return MMBO_OK;
 }
 
@@ -613,6 +711,20 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
                 }
             }
         }
+        // The entry point that allocates nothing holds kScratchPartialBytes of partial sums: where the pick's GlobalSplitU
+        // needs more, the same tile runs with the largest split that fits (down to none), so that every shape still
+        // runs under MMBO_CONFIG_AUTO.  (A config the caller names is taken as named, or refused.)
+        if (!f64 && ws_source == WsSource::kStatic) {
+            const ConfigRef c = config_ref(config_id);
+            int si = split_index(c.split);
+            auto fits = [&](int sidx) {
+                if (kSplits[sidx] == 1) return true;
+                if ((double)kSplits[sidx] * batch * (double)m * (double)n * sizeof(float) > (double)kScratchPartialBytes) return false;
+                return !c.ring || ring_shape_ok(dtype, c.tile, kSplits[sidx], transA, transB, m, n, k, c.x16);
+            };
+            while (si > 0 && !fits(si)) --si;
+            config_id = c.x16 ? x16_config_id(c.tile, si) : c.ring ? ring_config_id(c.tile, si) : staged_config_id(c.tile, si);
+        }
         if (!tile_span_ok(config_tile(dtype, config_id), transA, transB, lda, ldb, esz_in)) {
             // enormous leading dimensions: the first staged tile (no split-K) whose span fits, large tiles first
             const int ntiles = f64 ? NUM_F64_TILES : NUM_TILES;
@@ -668,9 +780,9 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
     // Split-K: the partial sums go to the stream's own workspace (or the static one), and both launches that use it (the
-    // GEMM and the reduction, which adds the splits in ascending order) are queued before the lock on the workspace
-    // table is given up.
-    std::unique_lock<std::mutex> ws_lock;
+    // GEMM and the reduction, which adds the splits in ascending order) are queued before the hold on that workspace
+    // is given up.
+    WsHold ws_hold;
     if (split > 1) {
         const size_t bytes = (size_t)split * batch * m * n * sizeof(float);
         char *base = nullptr;
@@ -679,8 +791,7 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
             int rc = static_scratch(&base);
             if (rc != MMBO_OK) return rc;
         } else {
-            ws_lock = std::unique_lock<std::mutex>(g_ws_mutex);
-            int rc = workspace(s, bytes, &base);
+            int rc = workspace(s, bytes, ws_hold, &base);
             if (rc != MMBO_OK) return rc;
         }
         a.ws = reinterpret_cast<float *>(base);

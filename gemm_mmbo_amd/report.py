@@ -11,7 +11,10 @@ peak, with rocBLAS's result as the check, :110-117).  This is that driver for th
                                                             # dtype s|h|d, ta/tb N|T;  e.g.  h,N,N,4096,128,4096
     options:  --json FILE (one JSON object per line)   --csv FILE   --reps R (timed groups, default 10)
               --inner I (launches per group; default: enough for about 2 ms)   --config ID (default: the automatic pick)
-              --no-check   --print-profile-commands
+              --no-check   --print-profile-commands   --ceilings
+    python -m gemm_mmbo_amd.report capture CASE --out DIR [--summary FILE]    # run the case under rocprofv3, pass by pass
+    python -m gemm_mmbo_amd.report summarise CASE DIR [--summary FILE]        # rocprofv3's CSV files -> text (no GPU needed)
+    python -m gemm_mmbo_amd.report cases                                      # (gemm_mmbo_amd/profiles.py)
 
 Per shape: GPU milliseconds per launch (median, minimum and maximum over the groups, HIP events on the launch stream),
 TFLOP/s, fraction of the matrix peak, the roofline bound min(peak, arithmetic intensity x 8 TB/s) and the fraction of it,
@@ -31,7 +34,7 @@ import sys
 PEAK_TFLOPS = {"h": 2500.0, "s": 157.3, "d": 78.6}         # MI355X dense matrix peaks: fp16, fp32, fp64
 HBM_TBPS = 8.0
 ESZ = {"h": 2, "s": 4, "d": 8}
-FIELDS = ["dtype", "transA", "transB", "m", "n", "k", "batch", "lda", "ldb", "ldc", "alpha", "beta", "config_id", "config",
+FIELDS = ["spec", "calls_total", "calls_timed", "dtype", "transA", "transB", "m", "n", "k", "batch", "lda", "ldb", "ldc", "alpha", "beta", "config_id", "config",
           "gpu_ms_median", "gpu_ms_min", "gpu_ms_max", "groups", "launches_per_group", "tflops", "frac_of_peak", "bound",
           "bound_tflops", "frac_of_bound", "algorithmic_bytes", "algorithmic_GBps", "frac_of_hbm_peak", "max_rel_err",
           "checked_against"]
@@ -98,6 +101,13 @@ def run_shape(G, torch, shape, reps, inner, config, check, seed=1):
         G.gemm_strided_batched(dt, ita, itb, m, n, k, alpha, a, lda, m * k, b, ldb, k * n, beta, c, ldc, ldc * n, batch, cfg,
                                stream)
 
+    calls = [0]                              # GEMM calls made for this shape with the config under test (for trace readers)
+    plain_launch = launch
+
+    def launch():
+        calls[0] += 1
+        plain_launch()
+
     launch()
     torch.cuda.synchronize()
     rel, against = None, None
@@ -127,7 +137,8 @@ def run_shape(G, torch, shape, reps, inner, config, check, seed=1):
     flops, nbytes, bound, bound_tf = roofline(d, m, n, k, batch, beta)
     tf = flops / med * 1e-9
     gbps = nbytes / med * 1e-6
-    return {"dtype": d, "transA": ta, "transB": tb, "m": m, "n": n, "k": k, "batch": batch, "lda": lda, "ldb": ldb, "ldc": ldc,
+    return {"spec": spec_of(shape), "calls_total": calls[0], "calls_timed": reps * inner,
+            "dtype": d, "transA": ta, "transB": tb, "m": m, "n": n, "k": k, "batch": batch, "lda": lda, "ldb": ldb, "ldc": ldc,
             "alpha": alpha, "beta": beta, "config_id": cid, "config": name, "gpu_ms_median": round(med, 5),
             "gpu_ms_min": round(per[0], 5), "gpu_ms_max": round(per[-1], 5), "groups": reps, "launches_per_group": inner,
             "tflops": round(tf, 2), "frac_of_peak": round(tf / PEAK_TFLOPS[d], 4), "bound": bound,
@@ -182,6 +193,10 @@ def profile_commands(shape):
 
 
 def main(argv=None):
+    argv = sys.argv[1:] if argv is None else list(argv)
+    if argv and argv[0] in ("capture", "summarise", "cases"):
+        from . import profiles
+        return profiles.main(argv)
     ap = argparse.ArgumentParser(prog="python -m gemm_mmbo_amd.report", description=__doc__.split("\n\n")[0])
     ap.add_argument("mode", choices=["configs", "hpl", "shapes"])
     ap.add_argument("specs", nargs="*")
@@ -193,6 +208,8 @@ def main(argv=None):
     ap.add_argument("--step", type=int, default=3840, help="hpl: step of M (the reference's run.sh uses 384)")
     ap.add_argument("--no-check", action="store_true")
     ap.add_argument("--print-profile-commands", action="store_true")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="finish with one record of what a register-only MFMA loop sustains on this box right now")
     args = ap.parse_args(argv)
     if args.reps < 1:
         ap.error("--reps must be at least 1")
@@ -232,6 +249,16 @@ def main(argv=None):
             for c in profile_commands(shape):
                 print("# " + c)
         torch.cuda.empty_cache()
+    if args.ceilings:
+        ceil = {}
+        for name, dt in (("f16", G.F16), ("f32", G.F32), ("f64", G.F64)):
+            for rnd in (0, 1):
+                tf, mhz = G.probe_mfma_ceiling(dt, bool(rnd))
+                ceil[f"{name}_{'random' if rnd else 'ones'}_operands"] = {"tflops": round(tf, 1), "shader_mhz": round(mhz)}
+        line = json.dumps({"mfma_issue_ceiling": ceil})
+        print(line, flush=True)
+        if jf:
+            jf.write(line + "\n")
     for f in (jf, cf):
         if f:
             f.close()

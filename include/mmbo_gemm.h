@@ -140,7 +140,9 @@ int mmbo_batch_xcd_remap(unsigned linear_id, unsigned tiles, unsigned batch, uns
  * of the library's device image (mmbo_static_workspace_bytes() bytes of partial sums, 32 MiB, held by every GPU the
  * library runs on until the process ends) instead of in memory from hipMalloc, and the call makes no hipMalloc, hipFree
  * or other allocating call.  A call whose partial sums (GlobalSplitU x batch x m x n x 4 bytes; mmbo_config_info of
- * mmbo_select_config's pick gives GlobalSplitU) do not fit is refused with MMBO_ERR_WORKSPACE and launches nothing;
+ * mmbo_select_config's pick gives GlobalSplitU) do not fit is refused with MMBO_ERR_WORKSPACE and launches nothing
+ * when the caller named the config; under MMBO_CONFIG_AUTO the picked tile then runs with the largest GlobalSplitU
+ * whose partial sums fit (down to none), so every shape runs under MMBO_CONFIG_AUTO here as well;
  * configs without split-K need no workspace and always run.  All calls on one GPU share that GPU's array: two such
  * split-K calls that overlap in time on one GPU (different streams, or different host threads) race on it -- keep them
  * on one stream.  The first call on a device looks the array's address up (hipGetSymbolAddress), once. */
@@ -153,8 +155,20 @@ size_t mmbo_static_workspace_bytes(void);
 
 /* Release the split-K workspaces held for the current device (one per stream that ran a split-K config; allocated
  * lazily, grown on demand, reused across calls).  Waits for the device.  The reference never frees what it loads
- * (src/gemm/driver.h:41). */
+ * (src/gemm/driver.h:41).
+ * The library keeps at most 8 such workspaces per device: a split-K call on a ninth stream retires the least recently
+ * used one (it then waits for the device once).  A workspace is keyed by the stream handle and by the device that is
+ * current at the call (make the stream's device current, as for any launch). */
 int mmbo_release_workspace(void);
+
+/* Release the workspace of one stream of the current device; waits for that stream only.  Call it before destroying
+ * a stream that ran split-K configs when the memory should come back at once (otherwise the slot is retired when eight
+ * other streams have needed one, or by mmbo_release_workspace).  A stream without a workspace is not an error. */
+int mmbo_release_stream_workspace(void *stream);
+
+/* How many split-K workspaces the library holds for the current device, and their total bytes (either pointer may
+ * be null).  A diagnostic; no counterpart in the reference. */
+int mmbo_workspace_info(size_t *slots, size_t *bytes);
 
 /* Measures what the MFMA pipes of the current device sustain with nothing else running: a register-only loop
  * of v_mfma_f32_16x16x32_f16 (MMBO_F16), v_mfma_f32_32x32x2_f32 (MMBO_F32) or v_mfma_f64_16x16x4_f64 (MMBO_F64) -- the

@@ -515,6 +515,45 @@ def test_split_k_on_two_streams_at_the_same_time():
             assert np.array_equal(first.view(np.uint8), outs[i][rep].cpu().numpy().view(np.uint8))
 
 
+def test_split_k_workspaces_stay_bounded_over_many_short_lived_streams():
+    """The library keeps one split-K workspace per stream, at most eight per device: a process that keeps creating and
+    destroying streams does not keep one buffer per stream handle it ever used (the launcher this replaces never frees
+    anything, src/gemm/driver.h:41).  Results stay those of the first call bit for bit; a stream's slot can be handed
+    back by name; release_workspace empties the table."""
+    import torch
+    import gemm_mmbo_amd as G
+    G.release_workspace()
+    assert G.workspace_info() == (0, 0)
+    p = U.Problem(F16, 0, 0, 1024, 128, 2048, 1.0, 0.0, seed=83, c_fill="nan")
+    cid = [c for c in range(G.num_configs(F16)) if G.config_info(F16, c)["split_k"] == 4 and G.config_info(F16, c)["macro_tile_m"] == 64][0]
+    dA, dB = torch.from_numpy(p.A).cuda(), torch.from_numpy(p.B).cuda()
+    first = None
+    most = 0
+    for i in range(64):
+        st = torch.cuda.Stream()
+        dC = torch.from_numpy(p.C).cuda()
+        st.wait_stream(torch.cuda.current_stream())
+        G.gemm(F16, 0, 0, p.m, p.n, p.k, 1.0, dA, p.lda, dB, p.ldb, 0.0, dC, p.ldc, cid, st)
+        st.synchronize()
+        out = dC.cpu().numpy()
+        if first is None:
+            first = out
+            U.check(p, first, "first short-lived stream")
+        else:
+            assert np.array_equal(first.view(np.uint8), out.view(np.uint8)), i
+        slots, nbytes = G.workspace_info()
+        most = max(most, slots)
+        assert 1 <= slots <= 8 and nbytes >= 4 * p.m * p.n * 4 * slots, (i, slots, nbytes)
+        if i % 16 == 5:
+            G.release_stream_workspace(st)              # hand this stream's slot back before the stream goes away
+            assert G.workspace_info()[0] == slots - 1
+        del st
+    assert most >= 2                                    # (distinct stream handles did get distinct slots)
+    G.release_stream_workspace(torch.cuda.Stream())     # a stream without a workspace: not an error
+    G.release_workspace()
+    assert G.workspace_info() == (0, 0)
+
+
 def test_every_shape_of_the_tuned_table_under_the_automatic_pick():
     """Each exact-shape row of csrc/tuned_table.hpp names a config by id: run the row's shape through MMBO_CONFIG_AUTO
     against the oracle, so a row that points at a config that cannot take its shape, or computes it wrongly, is found.
