@@ -18,7 +18,7 @@ LIB = os.path.join(CSRC, "libmmbo_gemm.so")
 NUM_TILES = 6  # keep in step with csrc/configs.hpp
 NUM_RING_TILES = 4
 NUM_F64_TILES = 6
-NUM_X16_TILES = 5
+NUM_X16_TILES = 8
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

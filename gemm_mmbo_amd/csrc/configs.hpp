@@ -66,13 +66,17 @@ constexpr int ring_bk(int dtype) { return dtype == 0 ? 16 : 32; }
 // Tiles of the 16x16-block ring kernel with accumulation-register accumulators (gemm_x16.hpp), both element types;
 // depthU is 32 (fp16) / 16 (fp32).
 // Config ids continue after the ring ones:  x16_tile + NUM_X16_TILES * split_index.
-constexpr int NUM_X16_TILES = 5;
+constexpr int NUM_X16_TILES = 8;
 constexpr RingRow kX16Tiles[NUM_X16_TILES] = {
     {256, 256, 2, 2, 5},     // four wavefronts of 128 x 128: 256 accumulator registers per lane, one work-group per CU
     {256, 256, 4, 2, 5},     // eight wavefronts of 64 x 128
     {128, 128, 2, 2, 5},     //  80 KB of LDS, two work-groups per CU
     {128,  64, 2, 2, 6},     //  72 KB, two per CU
     { 64,  64, 2, 2, 6},     //  48 KB, three per CU
+    {192, 192, 2, 2, 6},     // four wavefronts of 96 x 96, 144 KB: for sizes whose 256 x 256 tiles would leave a round of the
+                             // 256 CUs part empty (3000^2 is 144 tiles of 256 x 256 but 256 tiles of 192 x 192)
+    {256, 192, 2, 2, 5},     // four wavefronts of 128 x 96, 140 KB: the steps between 192 x 192 and 256 x 256
+    {192, 256, 2, 2, 5},     // four wavefronts of 96 x 128
 };
 
 // Config ids (fp32 and fp16 share them): [0, kStagedConfigs) the staged kernel's (tile, split) pairs, then the ring

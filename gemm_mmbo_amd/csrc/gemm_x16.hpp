@@ -104,6 +104,9 @@ __device__ __forceinline__ float acc_read()
 //     block, four consecutive k-rows x 32 bytes; its blocks sit 8 k-rows apart.  The chunk index is XORed with a
 //     mask of k so that the four k-rows of a block fall into different 64-byte groups and the two blocks served
 //     in one pass into different halves of a group.
+//     A tile whose row count is not a power of two (192) is laid out as NSUB sub-tiles of SUB rows, SUB the largest
+//     power of two that divides R: a 1 KB direct load fills whole k-rows of ONE sub-tile, the sub-tiles of a slice
+//     follow each other in LDS, and each is swizzled like a tile of SUB rows (16-row MFMA blocks never straddle two).
 template <typename T, bool KC, int R, int NW>
 struct Tile {
     static constexpr int ESZ = sizeof(T);
@@ -111,10 +114,16 @@ struct Tile {
     static constexpr int INSTRS = R / 16;
     static_assert(INSTRS % NW == 0, "tile must split evenly over the wavefronts");
     static constexpr int LPW = INSTRS / NW;
-    static constexpr int ROW_BYTES = R * ESZ;
+    static constexpr int SUB = KC ? R : (R & -R);                 // rows of a sub-tile (RC operands; the whole tile when R is a power of two)
+    static constexpr int NSUB = R / SUB;
+    static constexpr int ROW_BYTES = SUB * ESZ;                   // one k-row of one sub-tile
     static constexpr int CPR = ROW_BYTES / 16;
     static constexpr int KPI = 1024 / ROW_BYTES;
-    static_assert(KC || R == 64 || R == 128 || R == 256, "RC tile: a k-row is 128 to 1024 bytes, a power of two");
+    static constexpr int SUB_BYTES = SUB * 64;                    // one sub-tile of one slice
+    static constexpr int IPS = INSTRS / NSUB;                     // direct loads per sub-tile
+    static_assert(KC || (ROW_BYTES >= 64 * ESZ && ROW_BYTES <= 1024 && (ROW_BYTES & (ROW_BYTES - 1)) == 0),
+                  "RC tile: a k-row of a sub-tile is 64 elements to 1024 bytes, a power of two");
+    static_assert(KC || IPS * 1024 == SUB_BYTES, "a sub-tile is a whole number of 1 KB loads");
 
     __device__ static inline uint32_t rc_mask(uint32_t k)
     {
@@ -126,7 +135,12 @@ struct Tile {
     }
     __device__ static inline uint32_t kc_swz(uint32_t row) { return (row >> 1) & 3; }
     __device__ static inline uint32_t kc_off(uint32_t row, uint32_t chunk) { return row * 64 + ((chunk ^ kc_swz(row)) << 4); }
-    __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk) { return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4); }
+    // LDS offset of 16-byte group `chunk` (counted along all R rows) of k-row k
+    __device__ static inline uint32_t rc_off(uint32_t k, uint32_t chunk)
+    {
+        if constexpr (NSUB == 1) return k * ROW_BYTES + ((chunk ^ rc_mask(k)) << 4);
+        else return (chunk / CPR) * SUB_BYTES + k * ROW_BYTES + (((chunk % CPR) ^ rc_mask(k)) << 4);
+    }
 
     static constexpr uint32_t EPC = 16 / ESZ;                   // elements per 16-byte group
 
@@ -153,8 +167,8 @@ struct Tile {
             uint32_t chunk = (lane & 3) ^ kc_swz(row);
             return min(row, valid - 1) * ld * ESZ + chunk * 16;
         } else {
-            uint32_t k = q * KPI + lane / CPR;
-            uint32_t chunk = (lane % CPR) ^ rc_mask(k);
+            uint32_t k = (q % IPS) * KPI + lane / CPR;
+            uint32_t chunk = (q / IPS) * CPR + ((lane % CPR) ^ rc_mask(k));
             return k * ld * ESZ + rc_group_off(chunk, valid, back);
         }
     }
@@ -186,8 +200,8 @@ struct Tile {
                     v = u.v;
                 }
             } else {
-                uint32_t k = q * KPI + lane / CPR;
-                uint32_t chunk = (lane % CPR) ^ rc_mask(k);
+                uint32_t k = (q % IPS) * KPI + lane / CPR;
+                uint32_t chunk = (q / IPS) * CPR + ((lane % CPR) ^ rc_mask(k));
                 if (k < k_tail) v = *reinterpret_cast<const u32x4 *>(g + k * ld * ESZ + rc_group_off(chunk, valid, back));
             }
             *reinterpret_cast<u32x4 *>(dst + q * 1024 + lane * 16) = v;
@@ -267,6 +281,8 @@ struct Frags {
 
 // How many of a slice's `loads` direct loads have gone out before MFMA slot `slot` of `slots`: load l goes out after MFMA
 // number (2l+1) * slots / (2 * loads), evenly spaced, none first or last.
+constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
+
 constexpr int loads_before_slot(int loads, int slots, int slot)
 {
     const int l = (2 * loads * slot + slots) / (2 * slots);
@@ -618,8 +634,7 @@ gemm_x16_kernel(const GemmArgs args)
         auto tail_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             constexpr int par = decltype(PAR)::value;
             constexpr int LOP = par == 0 ? LA : LB;
-            constexpr int G = LA < LB ? LA : LB;                         // every count below is a multiple of the smaller LPW
-            static_assert(LA % G == 0 && LB % G == 0, "loads per slice of one operand must divide the other's");
+            constexpr int G = gcd_of(LA, LB);                            // every count below is a multiple of it
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
             mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf);

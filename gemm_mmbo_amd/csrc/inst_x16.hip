@@ -31,10 +31,10 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
         if (e != hipSuccess) return e;
         attr_set[dev].store(true, std::memory_order_release);
     }
-    // 256 x 256 tiles (one work-group per CU fits): on grids with more tiles than CUs the work-groups stay resident and
-    // walk the tiles themselves
+    // Tiles of which one work-group per CU fits (256 x 256, 192 x 192): on grids with more tiles than CUs the work-groups
+    // stay resident and walk the tiles themselves
     unsigned gx = args.nwg0 * args.nwg1;
-    if (R.bm == 256 && R.bn == 256) {
+    if (Cfg::LDS_BYTES > 80 * 1024) {
         static std::atomic<int> cus[64];
         int n = dev >= 0 && dev < 64 ? cus[dev].load(std::memory_order_acquire) : 0;
         if (n == 0) {

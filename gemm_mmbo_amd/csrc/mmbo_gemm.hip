@@ -485,16 +485,9 @@ static bool tile_span_ok(const TileRow &r, int transA, int transB, size_t lda, s
 // so every request of the direct loads touches one line more.  Measured on fp16: the 128 x 128 and smaller tiles, which
 // are bound by that stream, lose 13-26 % of their in-loop rate (3000^3 against 3072^3, 4104^3 against 4096^3, 8200 against
 // 8192), the 256 x 256 tile up to 15 % at 3000 and nothing at 4104 or 8200; fp32 tiles, MFMA-bound, lose nothing.
-static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, size_t n, size_t k, int batch,
-                              bool split_lines = false)
+static double model_time_tile(int dtype, const RingRow &r, double e, int split, size_t m, size_t n, size_t k, int batch)
 {
-    static const double eff[2][2][NUM_RING_TILES] = {
-        // 256x256 128x128 128x64  64x64
-        {{0.9451, 0.9134, 0.8667, 0.9015}, {0.9387, 0.9039, 0.8402, 0.8561}},       // fp32: ring, x16
-        {{0.5607, 0.3426, 0.2795, 0.2658}, {0.5879, 0.4873, 0.3151, 0.2560}},       // fp16: ring, x16
-    };
     const double launch = 5.9, fill = 0.65, c_us_per_kb = 0.0272, reduce_launch = 1.43, reduce_us_per_mb = 0.28;
-    const RingRow &r = kRingTiles[rt];                     // the x16 tiles of the same macro tile have the same depth
     const double esz = dtype == MMBO_F32 ? 4.0 : 2.0;
     const double flop_per_us_cu = dtype == MMBO_F32 ? 0.614e6 : 9.83e6;             // matrix peak of one CU
     const int bk = ring_bk(dtype);
@@ -505,8 +498,6 @@ static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, 
     const double cus = 256.0;
     const double wgs = (double)ceil_div(m, (size_t)r.bm) * (double)ceil_div(n, (size_t)r.bn) * split * batch;
     const double slices = std::ceil(std::ceil((double)k / bk) / split);
-    double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
-    if (split_lines && dtype == MMBO_F16) e *= rt == 0 ? 0.95 : 0.78;
     auto tile_time = [&](double resident) {
         return fill + slices * (2.0 * r.bm * r.bn * bk / flop_per_us_cu) * resident / e +
                c_us_per_kb * r.bm * r.bn * esz * resident / 1e3;
@@ -514,9 +505,39 @@ static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, 
     const double slots = cus * per_cu;
     const double full = std::floor(wgs / slots), last = wgs - full * slots;
     double t = launch + full * tile_time(per_cu);
-    if (last > 0) t += tile_time(std::ceil(last / cus));
+    if (last > 0) {
+        // A last round that leaves CUs idle runs faster per tile on fp16: the chip is power-limited on these MFMAs and the
+        // clock rises when fewer CUs draw power (HGEMM 3072^3 on 144 tiles of 256 x 256: 54 us against 74 us for a full
+        // round of the same tiles; 5120^3, 256 + 144 tiles: the second round takes 0.82 of the first).
+        const double busy = last >= cus ? 1.0 : last / cus;
+        const double boost = dtype == MMBO_F16 ? 0.45 + 0.55 * busy : 1.0;
+        t += tile_time(std::ceil(last / cus)) * boost;
+    }
     if (split > 1) t += reduce_launch + reduce_us_per_mb * (double)m * n * batch * (split * 4.0 + esz) / 1e6;
     return t;
+}
+static double model_time_ring(int dtype, bool x16, int rt, int split, size_t m, size_t n, size_t k, int batch,
+                              bool split_lines = false)
+{
+    static const double eff[2][2][NUM_RING_TILES] = {
+        // 256x256 128x128 128x64  64x64
+        {{0.9451, 0.9134, 0.8667, 0.9015}, {0.9387, 0.9039, 0.8402, 0.8561}},       // fp32: ring, x16
+        {{0.5607, 0.3426, 0.2795, 0.2658}, {0.5879, 0.4873, 0.3151, 0.2560}},       // fp16: ring, x16
+    };
+    double e = eff[dtype == MMBO_F32 ? 0 : 1][x16 ? 1 : 0][rt];
+    if (split_lines && dtype == MMBO_F16) e *= rt == 0 ? 0.95 : 0.78;
+    return model_time_tile(dtype, kRingTiles[rt], e, split, m, n, k, batch);      // the x16 tiles of the same macro tile have the same depth
+}
+// The x16 kernel's tiles without a ring-kernel twin: 192 x 192, 256 x 192, 192 x 256 (kX16Tiles[5..7]).  In-loop
+// efficiency: 192 x 192 from HGEMM 6144^3 (four whole rounds, 381 us) and SGEMM 3072^3 (one round, 404 us); the two
+// rectangular ones between that and the 256 x 256 tile's.
+constexpr int kFirstX16OnlyTile = 5;
+static double model_time_x16_only(int dtype, int tile, int split, size_t m, size_t n, size_t k, int batch, bool split_lines)
+{
+    static const double eff16[3] = {0.50, 0.55, 0.55}, eff32[3] = {0.93, 0.935, 0.935};
+    double e = (dtype == MMBO_F32 ? eff32 : eff16)[tile - kFirstX16OnlyTile];
+    if (split_lines && dtype == MMBO_F16) e *= 0.90;
+    return model_time_tile(dtype, kX16Tiles[tile], e, split, m, n, k, batch);
 }
 
 // The cost model's pick among the staged configs (fp32/fp16), which take any shape and any alignment.
@@ -588,6 +609,22 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
                     pick = x16 ? x16_config_id(x16_of_ring[rt], si) : ring_config_id(rt, si);
                 }
             }
+        // the 192-row and 192-column tiles: where they fill the rounds of 256 CUs better than the power-of-two tiles do
+        static_assert(kX16Tiles[kFirstX16OnlyTile].bm == 192 && kX16Tiles[kFirstX16OnlyTile].bn == 192 && NUM_X16_TILES == 8,
+                      "x16 tiles 5, 6, 7 are 192 x 192, 256 x 192, 192 x 256");
+        for (int tile = kFirstX16OnlyTile; tile < NUM_X16_TILES; ++tile) {
+            if (m < (size_t)kX16Tiles[tile].bm || n < (size_t)kX16Tiles[tile].bn) continue;
+            for (int si = 0; si < NUM_SPLITS; ++si) {
+                if (!ring_shape_ok(dtype, tile, kSplits[si], transA, transB, m, n, k, true)) continue;
+                if (kSplits[si] > 1 && (k / ring_bk(dtype)) / (size_t)kSplits[si] < 2) continue;
+                if ((size_t)batch * kSplits[si] > 65535) continue;
+                const double t = model_time_x16_only(dtype, tile, kSplits[si], m, n, k, batch, split_lines);
+                if (pick < 0 || t < pick_t) {
+                    pick_t = t;
+                    pick = x16_config_id(tile, si);
+                }
+            }
+        }
         if (pick >= 0) return pick;
     }
     return select_staged(dtype, m, n, k, batch);
@@ -767,7 +804,8 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
     a.splits = (uint32_t)split;
     a.k_per_split = (uint32_t)(split > 1 ? k_per_split : (k ? k : 1));
     a.batch = (uint32_t)batch;
-    a.chip_block = cref.x16 && r.bm == 256 && r.bn == 256 && nwg0 >= 16 && nwg1 >= 16;
+    // (tiles that run one work-group per CU: 256 x 256 and 192 x 192)
+    a.chip_block = cref.x16 && rr.depth * (rr.bm + rr.bn) * 64 > 80 * 1024 && nwg0 >= 16 && nwg1 >= 16;
     // batches of problems of at most 32 tiles (an XCD's CUs hold them at one time): each problem on one XCD
     a.batch_xcd = split == 1 && batch >= a.nxcd && batch % a.nxcd == 0 && nwg0 * nwg1 <= 32;
     auto aligned16 = [&](const void *p, size_t ld, long long stride) {

@@ -19,7 +19,7 @@ struct TunedRow {
 };
 
 // Ring tiles (kRingTiles): 0 = 256x256, 1 = 128x128, 2 = 128x64, 3 = 64x64; x16 tiles (kX16Tiles): 0 = 256x256 on four
-// wavefronts, 1 = on eight, 2 = 128x128, 3 = 128x64, 4 = 64x64.  The ids are built from (tile, GlobalSplitU), so a row
+// wavefronts, 1 = on eight, 2 = 128x128, 3 = 128x64, 4 = 64x64, 5 = 192x192, 6 = 256x192, 7 = 192x256.  The ids are built from (tile, GlobalSplitU), so a row
 // keeps its meaning when a tile or a split factor is added to the tables.
 constexpr int ring_id(int tile, int split) { return ring_config_id(tile, split_index(split)); }
 constexpr int x16_id(int tile, int split) { return x16_config_id(tile, split_index(split)); }
@@ -46,7 +46,7 @@ constexpr TunedRow kTuned[] = {
     {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // fp64 ids are rows of kTilesF64; the reference's HPL trailing update (src/gemm/run.sh:2-5)
     {2, 0, 0, 8192, 8192, 8192, 1, 0, 69.7f},
 };
-static_assert(ring_id(3, 1) == 33 && ring_id(3, 2) == 37 && x16_id(0, 1) == 50 && x16_id(4, 16) == 74,
-              "config id layout: 30 staged ids, 20 ring ids, 25 x16 ids");
+static_assert(ring_id(3, 1) == 33 && ring_id(3, 2) == 37 && x16_id(0, 1) == 50 && x16_id(7, 16) == 89,
+              "config id layout: 30 staged ids, 20 ring ids, 40 x16 ids");
 
 }  // namespace mmbo

@@ -99,7 +99,7 @@ def test_batches_of_small_problems_one_per_xcd():
                 ran += 1
     assert ran >= 60
     for (dtype, m, n, k, batch, cid) in ((F16, 256, 256, 256, 12, -1), (F16, 384, 384, 128, 8, _x16_ids(F16)[4]),
-                                         (F32, 128, 128, 512, 8, _x16_ids(F32)[4 + 5])):
+                                         (F32, 128, 128, 512, 8, _x16_ids(F32)[4 + 8])):
         p = U.Problem(dtype, 1, 0, m, n, k, 1.0, 1.0, batch=batch, seed=3, dist="normal" if dtype == F16 else "uniform", c_fill="uniform")
         _run_and_check(p, cid, label=f"plain order {m}x{n}x{k} b{batch}")
 
@@ -126,7 +126,7 @@ def test_every_config_every_transpose_ragged(dtype, ta, tb):
             continue
         _run_and_check(p, cid, label=f"config {cid} {name}")
         taken += "MFMA16x16" in name
-    assert taken == 25
+    assert taken == 40
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -182,11 +182,11 @@ def test_ring_kernel_every_config_every_transpose(dtype, ta, tb):
 def test_x16_kernel_every_config_every_transpose(dtype, ta, tb):
     """The ring kernel on 16x16 MFMA blocks (v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x4_f32) with accumulators pinned
     to the accumulation registers, by explicit config id: every tile (4 and 8 wavefronts, 64 to 256 accumulator
-    registers) and split-K factor, K shorter and longer than the ring, odd slice counts (the paired-load schedule has an
+    registers, the 192 x 192 tile whose row-contiguous operands lie in LDS as three sub-tiles of 64 rows) and split-K factor, K shorter and longer than the ring, odd slice counts (the paired-load schedule has an
     even/odd rhythm), beta read-modify-write, batches."""
     import gemm_mmbo_amd as G
     ids = _x16_ids(dtype)
-    assert len(ids) == 25
+    assert len(ids) == 40
     bk = 16 if dtype == F32 else 32
     ran = 0
     for cid in ids:
@@ -200,7 +200,7 @@ def test_x16_kernel_every_config_every_transpose(dtype, ta, tb):
                           dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
             _run_and_check(p, cid, label=f"{d['name']} {m}x{n}x{k} b{batch}")
             ran += 1
-    assert ran == 125
+    assert ran == 200
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
@@ -247,7 +247,7 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
             _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch} ld {lda},{ldb}",
                            offsets=(0, 0, 0) if aligned else (1, 3, 1))
             ran += 1
-    assert ran >= 25 * 16
+    assert ran >= 40 * 16
 
 
 def test_x16_kernel_chip_block_order_and_refusals():
@@ -707,7 +707,7 @@ def test_offline_tuner_emits_table_rows_for_small_shapes():
                 fam, tile, split = re.match(r"(\w+)\((\d), (\d+)\)", t).groups()
                 assert (fam == "x16_id") == ("_ACC" in d["name"]) and int(split) == d["split_k"]
                 base = 50 if fam == "x16_id" else 30
-                ntile = 5 if fam == "x16_id" else 4
+                ntile = 8 if fam == "x16_id" else 4
                 assert cid == base + int(tile) + ntile * [1, 2, 4, 8, 16].index(int(split))
 
 

@@ -27,7 +27,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
 pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not installed")
 
 #        source file            defines
-UNITS = [("inst_x16.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(5)] + \
+UNITS = [("inst_x16.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(8)] + \
         [("inst_ring.hip", ["-DMMBO_DTYPE=%d" % d, "-DMMBO_TILE=%d" % t]) for d in (0, 1) for t in range(4)]
 
 
@@ -267,4 +267,4 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
-    assert seen == 40
+    assert seen == 64
