@@ -25,26 +25,26 @@ constexpr int ring_id(int tile, int split) { return ring_config_id(tile, split_i
 constexpr int x16_id(int tile, int split) { return x16_config_id(tile, split_index(split)); }
 
 constexpr TunedRow kTuned[] = {
-    //dtype ta tb m n k batch id TFLOP/s
-    {0, 0, 0, 1024, 1024, 1024, 1, ring_id(3, 1), 93.0f},
-    {0, 0, 1, 4096, 4096, 4096, 1, ring_id(0, 1), 140.2f},
-    {0, 1, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 145.0f},
-    {0, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 46.6f},
-    {1, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 82.4f},
-    {0, 0, 0, 4096, 128, 4096, 1, ring_id(3, 4), 95.0f},
-    {1, 0, 0, 4096, 128, 4096, 1, ring_id(3, 2), 272.2f},
-    {0, 0, 0, 128, 4096, 8192, 1, ring_id(3, 8), 108.8f},
-    {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 423.9f},
-    {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 442.8f},
-    {0, 0, 0, 2048, 2048, 2048, 1, ring_id(2, 1), 128.6f},
-    {1, 0, 0, 2048, 2048, 2048, 1, x16_id(2, 1), 761.2f},
-    {0, 0, 1, 44160, 2048, 384, 1, x16_id(2, 1), 120.5f},
-    {0, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 146.1f},
-    {1, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 1355.2f},
-    {0, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 143.6f},
-    {1, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 1245.0f},
-    {2, 0, 1, 44160, 2048, 384, 1, 2, 59.3f},      // fp64 ids are rows of kTilesF64; the reference's HPL trailing update (src/gemm/run.sh:2-5)
-    {2, 0, 0, 8192, 8192, 8192, 1, 0, 69.7f},
+    //dtype ta tb m n k batch id TFLOP/s (one tuner run on one MI355X; boxes differ by a few percent)
+    {0, 0, 0, 1024, 1024, 1024, 1, ring_id(3, 1), 99.2f},
+    {0, 0, 1, 4096, 4096, 4096, 1, ring_id(1, 1), 146.2f},
+    {0, 1, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 147.9f},
+    {0, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 52.2f},
+    {1, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 89.9f},
+    {0, 0, 0, 4096, 128, 4096, 1, ring_id(3, 4), 104.8f},
+    {1, 0, 0, 4096, 128, 4096, 1, ring_id(3, 2), 276.1f},
+    {0, 0, 0, 128, 4096, 8192, 1, ring_id(1, 8), 118.9f},
+    {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 425.8f},
+    {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 567.0f},
+    {0, 0, 0, 2048, 2048, 2048, 1, x16_id(3, 1), 132.6f},
+    {1, 0, 0, 2048, 2048, 2048, 1, x16_id(2, 1), 834.2f},
+    {0, 0, 1, 44160, 2048, 384, 1, ring_id(1, 1), 128.0f},
+    {0, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 149.8f},
+    {1, 0, 0, 8192, 8192, 8192, 1, x16_id(0, 1), 1453.7f},
+    {0, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 147.2f},
+    {1, 0, 0, 4096, 4096, 4096, 1, x16_id(0, 1), 1319.3f},
+    {2, 0, 1, 44160, 2048, 384, 1, 2, 60.3f},      // fp64 ids are rows of kTilesF64; the reference's HPL trailing update (src/gemm/run.sh:2-5)
+    {2, 0, 0, 8192, 8192, 8192, 1, 0, 70.0f},
 };
 static_assert(ring_id(3, 1) == 33 && ring_id(3, 2) == 37 && x16_id(0, 1) == 50 && x16_id(7, 16) == 89,
               "config id layout: 30 staged ids, 20 ring ids, 40 x16 ids");
