@@ -389,8 +389,8 @@ def summarise_shapes(case, outdir):
         for pname, counter, factor, word in (("fetch", "FETCH_SIZE", 2.0, "fetched"), ("write", "WRITE_SIZE", 1.0, "written")):
             if pname in extra:
                 sparts, cnt = extra[pname]
-                _, _, stimed = sparts[si]
-                per_call = sum(cnt.get(x["id"], {}).get(counter, 0.0) for x in stimed) / max(r["calls_timed"], 1)
+                prec, _, stimed = sparts[si]          # (each pass sizes its own groups: its own record says how many calls it timed)
+                per_call = sum(cnt.get(x["id"], {}).get(counter, 0.0) for x in stimed) / max(prec["calls_timed"], 1)
                 moved.append(f"{word} {per_call * 1024 * factor / 1e6:.1f} MB")
         if moved:
             L.append("   measured per GEMM (all its launches; FETCH_SIZE x 2.0, WRITE_SIZE x 1.0 -- the factors these counters read for a "
