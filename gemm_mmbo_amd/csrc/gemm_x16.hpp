@@ -311,6 +311,13 @@ struct X16Cfg {
     static constexpr int BATCH = TileA::LPW + TileB::LPW;         // direct loads per thread per slice
     static constexpr int NMFMA = FM * FN * MPF;
     static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
+    // Old C ahead of the epilogue (fp16, beta != 0): a wavefront's FM * FN / 2 sixteen-byte groups per lane (two vertically
+    // adjacent blocks each, as the epilogue reads them) are fetched with direct loads into the ring buffers the last
+    // slices no longer need, a quarter of them under each of the last four slices.
+    static constexpr int C_GROUPS = FM * FN / 2;
+    static constexpr int C_PER_SLICE = C_GROUPS / 4;
+    static constexpr bool C_PREFETCH = ESZ == 2 && FM % 2 == 0 && C_GROUPS % 4 == 0 && C_PER_SLICE * 8 == NMFMA &&
+                                       C_PER_SLICE * NW * 1024 <= SLICE_BYTES;
 };
 
 // PAIR: fetch two slices of one operand per iteration (see mfma_and_read); on when an operand is k-contiguous.
@@ -428,6 +435,21 @@ gemm_x16_kernel(const GemmArgs args)
     FragA fa[2];
     FragB fb[2];
 
+    // Old C ahead of the epilogue (Cfg::C_PREFETCH; paired mode, whole tiles, whole slices, at least DEPTH + 1 of them).
+    // Group q of this wavefront = blocks (i, j), (i + 1, j) with j = q / (FM / 2), i = 2 * (q % (FM / 2)): the lane's 16 bytes
+    // start at  C_tile + (lane's column * ldc + lane's row of the pair) + (j * 16 * ldc + i * 16)  elements -- the part in
+    // front is the lane's constant offset, the part behind a scalar offset of the load.  Group q goes to the ring buffer of
+    // slice n_slice - 4 + q / C_PER_SLICE (free from that slice's iteration on), at wave * C_PER_SLICE KB + (q % C_PER_SLICE) KB.
+    const bool c_ahead = Cfg::C_PREFETCH && PAIR && args.c_prefetch != 0 && m_here == (uint32_t)BM && n_here == (uint32_t)BN &&
+                         k_tail == 0 && n_slice >= DEPTH + 1;
+    // (set up whether used or not: a descriptor that is assigned under a branch ends up in vector registers, where a
+    // buffer load cannot take it)
+    [[maybe_unused]] const u32x4 curC = slice_cursor(uniform_address(
+        static_cast<const char *>(args.C) + ((int64_t)batch * args.strideC + (int64_t)col0 * args.ldc + row0) * ESZ));
+    [[maybe_unused]] const uint32_t c_lane_off =
+        ((wn * Cfg::TN + (lane & 15)) * args.ldc + wm * Cfg::TM + (((lane >> 4) & 1) ? 4 * (lane >> 4) + 12 : 4 * (lane >> 4))) * ESZ;
+    [[maybe_unused]] const uint32_t c_col_step = __builtin_amdgcn_readfirstlane(16 * args.ldc * ESZ);
+
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
         a.read_all(t, adA);
@@ -447,7 +469,8 @@ gemm_x16_kernel(const GemmArgs args)
     // (measured: half-line requests stream at 35-52 B/clk/CU from L2, whole lines at 72-91).  `load` / `load2`
     // say whether the first / second slice of the pair exists.
     auto mfma_and_read = [&](auto LOAD, auto PAR, const FragA &ca, const FragB &cb, FragA &na, FragB &nb, int nbuf, bool load,
-                             bool load2, int lbuf) {
+                             bool load2, int lbuf, auto OLD_C, int c_first) {
+        constexpr bool old_c = decltype(OLD_C)::value;            // this slice carries a quarter of the old C (no operand loads then)
         constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load` (and `load2`)
         constexpr int par = decltype(PAR)::value;
         constexpr int opn = par ^ EVEN_OP;                         // paired mode: the operand this iteration fetches
@@ -460,6 +483,9 @@ gemm_x16_kernel(const GemmArgs args)
         uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, lbuf), dst_b = op_dst(std::integral_constant<int, 1>{}, lbuf);
         if constexpr (load_mode != 0 && PAIR) asm volatile("" : "+s"(dst_x0), "+s"(dst_x1));
         if constexpr (load_mode != 0 && !PAIR) asm volatile("" : "+s"(dst_a), "+s"(dst_b));
+        // old C ahead of the epilogue: this iteration's groups c_first .. c_first + C_PER_SLICE - 1 go to buffer lbuf (the
+        // one this slice left; no operand load goes there any more), one after every eighth MFMA
+        [[maybe_unused]] const uint32_t c_dst = lds_base + (uint32_t)lbuf * Cfg::SLICE_BYTES + wave * (Cfg::C_PER_SLICE * 1024);
         uint32_t read_a[FragA::NADDR], read_b[FragB::NADDR];      // addresses of the LDS reads, each live from its first use to its last
         static_for<NMFMA>([&](auto M) {
             constexpr int m = decltype(M)::value;
@@ -521,12 +547,20 @@ gemm_x16_kernel(const GemmArgs args)
                     if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b, DESTINATION_SET);
                 }
             });
+            if constexpr (old_c && Cfg::C_PREFETCH && PAIR && m % 8 == 3) {
+                constexpr int c = m / 8;
+                const uint32_t q = (uint32_t)c_first + c;             // group q: column block q / (FM / 2), row-block pair q % (FM / 2)
+                const uint32_t soff = __builtin_amdgcn_readfirstlane((q / (FM / 2)) * c_col_step + (q % (FM / 2)) * (32 * ESZ));
+                direct_load16<true>(curC, soff, c_lane_off, c_dst + c * 1024);
+            }
             // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
             // pad the gap with an s_nop, which costs an issue slot like any other instruction)
             __builtin_amdgcn_sched_barrier(0);
         });
-        // the cursors move past what this iteration requested (past the end of k in the last iterations: never used again)
-        if constexpr (load_mode != 0 && PAIR) advance_op(std::integral_constant<int, opn>{}, 2);
+        // the cursors move past what this iteration requested (past the end of k in the last iterations: never used again).
+        // The paired tail moves them itself, behind its choice between two copies of the slice: a cursor that is changed on
+        // one side of a branch only comes out of the merge in vector registers, where a buffer load cannot take it.
+        if constexpr (load_mode == 1 && PAIR) advance_op(std::integral_constant<int, opn>{}, 2);
         if constexpr (load_mode != 0 && !PAIR) {
             advance(curA, (uint64_t)stepA);
             advance(curB, (uint64_t)stepB);
@@ -564,7 +598,7 @@ gemm_x16_kernel(const GemmArgs args)
         // steady state: every slice issues loads, no flag tests inside the MFMA stream
         auto steady_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-            mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, buf);
+            mfma_and_read(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, true, true, buf, std::false_type{}, 0);
             MMBO_WAIT_LGKM0();
             MMBO_WAIT_VM(BATCH * (DEPTH - 2));
             MMBO_BARRIER();
@@ -575,7 +609,7 @@ gemm_x16_kernel(const GemmArgs args)
         auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH < n_slice;
-            mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, buf);
+            mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, buf, std::false_type{}, 0);
             MMBO_WAIT_LGKM0();
             if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);
             MMBO_BARRIER();
@@ -623,7 +657,7 @@ gemm_x16_kernel(const GemmArgs args)
             constexpr int KEEP = own * ((DEPTH - 3 + 1) / 2) + other * ((DEPTH - 3) / 2);
             static_assert(KEEP < 64, "more loads in flight than vmcnt can count");
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-            mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, buf);
+            mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, buf, std::false_type{}, 0);
             MMBO_WAIT_LGKM0();
             MMBO_WAIT_VM(KEEP);
             MMBO_BARRIER();
@@ -637,11 +671,20 @@ gemm_x16_kernel(const GemmArgs args)
             constexpr int G = gcd_of(LA, LB);                            // every count below is a multiple of it
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
-            mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf);
+            // the last four slices carry the old C of the epilogue (no operand load is left to issue by then)
+            // (a copy of the slice of its own, chosen once per slice: a test in front of each of its loads cost the tails of
+            // short-k problems without C to fetch 1-3 %)
+            // (through readfirstlane: the choice below is then a scalar branch between two straight-line copies; left to the
+            // compiler's own view of what is uniform it became a lane-mask test with the two copies chained behind each other)
+            const int c_first = __builtin_amdgcn_readfirstlane((c_ahead && s + 4 >= n_slice) ? (s + 4 - n_slice) * Cfg::C_PER_SLICE : -1);
+            if (c_first >= 0) mfma_and_read(std::integral_constant<int, 0>{}, PAR, ca, cb, na, nb, nbuf, false, false, buf, std::true_type{}, c_first);
+            else mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf, std::false_type{}, 0);
+            advance_op(std::integral_constant<int, par ^ EVEN_OP>{}, 2);
             MMBO_WAIT_LGKM0();
-            const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP;
+            const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP + (c_first >= 0 ? Cfg::C_PER_SLICE : 0);
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
-            constexpr int KMAX = 2 * (LA > LB ? LA : LB) * 3;
+            constexpr int KMAX0 = 2 * (LA > LB ? LA : LB) * 3, KC3 = Cfg::C_PREFETCH ? 3 * Cfg::C_PER_SLICE : 0;
+            constexpr int KMAX = ((KMAX0 > KC3 ? KMAX0 : KC3) + G - 1) / G * G;
             bool waited = false;
             static_for<KMAX / G>([&](auto Q) {
                 constexpr int c = KMAX - decltype(Q)::value * G;          // KMAX, KMAX-G, ..., G
@@ -802,8 +845,33 @@ gemm_x16_kernel(const GemmArgs args)
     };
     if (vec_c && beta != 0.0f) {
         if constexpr (PAIRED_C) {
-            // the whole wave tile of old C is requested before its first value is used (see below)
+            // the whole wave tile of old C is requested before its first value is used (see below) -- or was requested
+            // under the last four slices and is waiting in the ring buffers those slices left (c_ahead)
             u32x4 cold[FM * FN / 2];
+            bool from_lds = false;
+            if constexpr (Cfg::C_PREFETCH && PAIR) {
+                if (c_ahead) {
+                    from_lds = true;
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's own loads: nobody else reads them
+                    const uint32_t first_buf = (uint32_t)(n_slice - 4) % DEPTH;
+                    const uint32_t mine = lds_base + wave * (Cfg::C_PER_SLICE * 1024) + lane * 16;
+                    static_for<4>([&](auto CC) {
+                        constexpr int cc = decltype(CC)::value;
+                        uint32_t b = first_buf + cc;
+                        if (b >= (uint32_t)DEPTH) b -= DEPTH;
+                        const uint32_t at = mine + b * Cfg::SLICE_BYTES;
+                        static_for<Cfg::C_PER_SLICE>([&](auto Q) {
+                            constexpr int q = decltype(Q)::value;
+                            cold[cc * Cfg::C_PER_SLICE + q] = lds_read_b128<q * 1024>(at);
+                        });
+                    });
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    // (a resident work-group's next tile sends its first loads into these buffers: not before every wavefront
+                    // has taken its old C out of them)
+                    __syncthreads();
+                }
+            }
+            if (!from_lds)
             static_for<FM * FN / 2>([&](auto IJ) {
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
                 cold[decltype(IJ)::value] = *reinterpret_cast<const u32x4 *>(C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16);

@@ -814,6 +814,10 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
     a.vec_a = aligned16(A, lda, strideA);
     a.vec_b = aligned16(B, ldb, strideB);
     a.vec_c = aligned16(C, ldc, strideC);
+    // beta != 0 on the x16 kernel's fp16 path: the old C of a tile is fetched into LDS under the tile's last slices (one
+    // tile's span of C, tile columns x ldc, must then fit the 32-bit offsets of a buffer load)
+    a.c_prefetch = cref.x16 && dtype == MMBO_F16 && beta_f != 0.0f && split == 1 && a.vec_c &&
+                   (size_t)r.bn * ldc * esz < 0x7FFFFF00ull;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;

@@ -67,28 +67,68 @@ def _vregs(text):
     return regs
 
 
+def _sregs(text):
+    regs = set()
+    for a, b in re.findall(r"\bs\[(\d+):(\d+)\]", text):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(a) for a in re.findall(r"\bs(\d+)\b", text))
+    return regs
+
+
 def _inflight_violations(body):
     """Forward data flow over the kernel's control-flow graph: the set of registers with an LDS read in flight at
     each instruction is the union over its predecessors; a read adds its destination, `s_waitcnt lgkmcnt(0)` empties
-    the set, and any other instruction that names a register of the set is a violation."""
+    the set, and any other instruction that names a register of the set is a violation.
+
+    The walk follows one kind of infeasible path no further: for `if (c) A else B` between two long straight-line
+    blocks the compiler emits "B (when !c), flag = 0 -- or flag = -1 -- then: A when flag", with the flag in a scalar
+    register pair (`s_mov_b64 s[a:b], 0` / `-1` ... `s_and_b64 vcc, exec, s[a:b]` ... `s_cbranch_vccz`).  The state
+    therefore carries the flags whose constant value is known on the path at hand, and a branch on such a flag has one
+    successor."""
     label = {t[:-1]: i for i, t in enumerate(body) if t.endswith(":")}
 
-    def succ(i, t):
+    def step_flags(t, flags, vcc):
+        """(flags, vcc) after instruction t.  flags: frozenset of ((lo, hi), value); vcc: None, 0 or 1."""
+        m = re.match(r"s_mov_b64 s\[(\d+):(\d+)\], (0|-1)$", t)
+        if m:
+            key = (int(m.group(1)), int(m.group(2)))
+            return frozenset({f for f in flags if f[0] != key} | {(key, 0 if m.group(3) == "0" else 1)}), vcc
+        m = re.match(r"s_and_b64 vcc, exec, s\[(\d+):(\d+)\]$", t)
+        if m:
+            key = (int(m.group(1)), int(m.group(2)))
+            return flags, next((v for k, v in flags if k == key), None)
+        if t.startswith(("s_", "v_cmp", "v_readlane", "v_readfirstlane")) and not t.startswith(("s_cbranch", "s_branch", "s_waitcnt", "s_nop", "s_barrier")):
+            dst = t.split(None, 1)[1].split(",")[0] if " " in t else ""
+            if "vcc" in dst or t.startswith("v_cmp"):
+                vcc = None
+            hit = _sregs(dst)
+            if hit:
+                flags = frozenset(f for f in flags if not (set(range(f[0][0], f[0][1] + 1)) & hit))
+        return flags, vcc
+
+    def succ(i, t, vcc):
         if t.startswith("s_endpgm"):
             return []
         m = re.match(r"s_(c?branch\w*) (\.LBB\w+)", t)
         if m:
             tgt = label[m.group(2)]
-            return [tgt] if m.group(1) == "branch" else [i + 1, tgt]
+            if m.group(1) == "branch":
+                return [tgt]
+            if vcc is not None and m.group(1) in ("cbranch_vccz", "cbranch_vccnz"):
+                taken = (vcc == 0) == (m.group(1) == "cbranch_vccz")
+                return [tgt] if taken else [i + 1]
+            return [i + 1, tgt]
         return [i + 1] if i + 1 < len(body) else []
 
-    pend_in = [None] * len(body)
-    pend_in[0] = frozenset()
-    work, bad = [0], {}
+    start = (0, frozenset(), None)
+    pend_in = {start: frozenset()}
+    work, bad = [start], {}
     while work:
-        i = work.pop()
-        t, cur = body[i], pend_in[i]
+        node = work.pop()
+        i, flags, vcc = node
+        t, cur = body[i], pend_in[node]
         out = cur
+        nflags, nvcc = flags, vcc
         if not t.endswith(":"):
             m = re.match(r"ds_read\w* (v\[\d+:\d+\]|v\d+),", t)
             if m:
@@ -99,11 +139,13 @@ def _inflight_violations(body):
                 out = frozenset()
             elif cur and (_vregs(t) & cur):
                 bad[i] = t
-        for j in succ(i, t):
-            new = out if pend_in[j] is None else pend_in[j] | out
-            if new != pend_in[j]:
-                pend_in[j] = frozenset(new)
-                work.append(j)
+            nflags, nvcc = step_flags(t, flags, vcc)
+        for j in succ(i, t, vcc):
+            nxt = (j, nflags, nvcc)
+            new = out if nxt not in pend_in else pend_in[nxt] | out
+            if nxt not in pend_in or new != pend_in[nxt]:
+                pend_in[nxt] = frozenset(new)
+                work.append(nxt)
     return [bad[i] for i in sorted(bad)]
 
 
@@ -112,6 +154,20 @@ def asm_files(tmp_path_factory):
     outdir = str(tmp_path_factory.mktemp("asm"))
     with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
         return list(ex.map(lambda u: _compile(u, outdir), UNITS))
+
+
+def test_checker_follows_a_constant_flag_but_not_an_unknown_one():
+    # "if (c) A else B" as the compiler lays it out: B, flag = 0, then A under the flag.  With the flag known the path from
+    # B's read into A does not exist; with the flag unknown (set from a comparison) it does, and A's use is a violation.
+    tail = ["s_and_b64 vcc, exec, s[6:7]", "s_cbranch_vccz .LBB0_9", "v_add_u32_e32 v11, s3, v9", ".LBB0_9:", "s_waitcnt lgkmcnt(0)", "s_endpgm"]
+    known = ["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], 0", ".LBB0_8:"] + tail
+    assert _inflight_violations(known) == []
+    unknown = ["ds_read_b128 v[10:13], v5 offset:64", "s_cselect_b64 s[6:7], -1, 0", ".LBB0_8:"] + tail
+    assert _inflight_violations(unknown) == ["v_add_u32_e32 v11, s3, v9"]
+    overwritten = ["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], 0", "s_or_b64 s[6:7], s[6:7], s[20:21]", ".LBB0_8:"] + tail
+    assert _inflight_violations(overwritten) == ["v_add_u32_e32 v11, s3, v9"]
+    set_one = ["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], -1", ".LBB0_8:"] + tail
+    assert _inflight_violations(set_one) == ["v_add_u32_e32 v11, s3, v9"]
 
 
 def test_checker_sees_a_planted_violation():
