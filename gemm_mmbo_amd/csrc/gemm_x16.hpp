@@ -324,11 +324,15 @@ struct X16Cfg {
 // EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
 // one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
+// OLD_C_AHEAD: the variant for beta != 0 that fetches a tile's old C into LDS under the tile's last four slices (see c_ahead
+// below).  A kernel of its own, chosen by the host: with the code in the one kernel, calls that have no C to read paid
+// 1.5-3 % on short-k and mid-size shapes for tails that had grown.
 template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, bool PAIR = (TA || !TB),
-          int EVEN_OP = (TA ? 0 : 1)>
+          int EVEN_OP = (TA ? 0 : 1), bool OLD_C_AHEAD = false>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_x16_kernel(const GemmArgs args)
 {
+    static_assert(!OLD_C_AHEAD || (PAIR && X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>::C_PREFETCH), "no old-C variant of this kernel");
     using namespace x16;
     using Cfg = X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>;
     using TileA = typename Cfg::TileA;
@@ -440,15 +444,15 @@ gemm_x16_kernel(const GemmArgs args)
     // start at  C_tile + (lane's column * ldc + lane's row of the pair) + (j * 16 * ldc + i * 16)  elements -- the part in
     // front is the lane's constant offset, the part behind a scalar offset of the load.  Group q goes to the ring buffer of
     // slice n_slice - 4 + q / C_PER_SLICE (free from that slice's iteration on), at wave * C_PER_SLICE KB + (q % C_PER_SLICE) KB.
-    const bool c_ahead = Cfg::C_PREFETCH && PAIR && args.c_prefetch != 0 && m_here == (uint32_t)BM && n_here == (uint32_t)BN &&
+    const bool c_ahead = OLD_C_AHEAD && args.c_prefetch != 0 && m_here == (uint32_t)BM && n_here == (uint32_t)BN &&
                          k_tail == 0 && n_slice >= DEPTH + 1;
     // (set up whether used or not: a descriptor that is assigned under a branch ends up in vector registers, where a
     // buffer load cannot take it)
     [[maybe_unused]] const u32x4 curC = slice_cursor(uniform_address(
-        static_cast<const char *>(args.C) + ((int64_t)batch * args.strideC + (int64_t)col0 * args.ldc + row0) * ESZ));
-    [[maybe_unused]] const uint32_t c_lane_off =
+        static_cast<const char *>(args.C) + (OLD_C_AHEAD ? ((int64_t)batch * args.strideC + (int64_t)col0 * args.ldc + row0) * ESZ : 0)));
+    [[maybe_unused]] const uint32_t c_lane_off = !OLD_C_AHEAD ? 0u :
         ((wn * Cfg::TN + (lane & 15)) * args.ldc + wm * Cfg::TM + (((lane >> 4) & 1) ? 4 * (lane >> 4) + 12 : 4 * (lane >> 4))) * ESZ;
-    [[maybe_unused]] const uint32_t c_col_step = __builtin_amdgcn_readfirstlane(16 * args.ldc * ESZ);
+    [[maybe_unused]] const uint32_t c_col_step = !OLD_C_AHEAD ? 0u : __builtin_amdgcn_readfirstlane(16 * args.ldc * ESZ);
 
     auto read_slice = [&](FragA &a, FragB &b, int buf) {
         const uint32_t t = lds_base + buf * Cfg::SLICE_BYTES;
@@ -547,7 +551,7 @@ gemm_x16_kernel(const GemmArgs args)
                     if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b, DESTINATION_SET);
                 }
             });
-            if constexpr (old_c && Cfg::C_PREFETCH && PAIR && m % 8 == 3) {
+            if constexpr (old_c && OLD_C_AHEAD && m % 8 == 3) {
                 constexpr int c = m / 8;
                 const uint32_t q = (uint32_t)c_first + c;             // group q: column block q / (FM / 2), row-block pair q % (FM / 2)
                 const uint32_t soff = __builtin_amdgcn_readfirstlane((q / (FM / 2)) * c_col_step + (q % (FM / 2)) * (32 * ESZ));
@@ -676,14 +680,19 @@ gemm_x16_kernel(const GemmArgs args)
             // short-k problems without C to fetch 1-3 %)
             // (through readfirstlane: the choice below is then a scalar branch between two straight-line copies; left to the
             // compiler's own view of what is uniform it became a lane-mask test with the two copies chained behind each other)
-            const int c_first = __builtin_amdgcn_readfirstlane((c_ahead && s + 4 >= n_slice) ? (s + 4 - n_slice) * Cfg::C_PER_SLICE : -1);
-            if (c_first >= 0) mfma_and_read(std::integral_constant<int, 0>{}, PAR, ca, cb, na, nb, nbuf, false, false, buf, std::true_type{}, c_first);
-            else mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf, std::false_type{}, 0);
+            const int c_first = !OLD_C_AHEAD ? -1 :
+                __builtin_amdgcn_readfirstlane((c_ahead && s + 4 >= n_slice) ? (s + 4 - n_slice) * Cfg::C_PER_SLICE : -1);
+            if constexpr (OLD_C_AHEAD) {
+                if (c_first >= 0) mfma_and_read(std::integral_constant<int, 0>{}, PAR, ca, cb, na, nb, nbuf, false, false, buf, std::true_type{}, c_first);
+                else mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf, std::false_type{}, 0);
+            } else {
+                mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf, std::false_type{}, 0);
+            }
             advance_op(std::integral_constant<int, par ^ EVEN_OP>{}, 2);
             MMBO_WAIT_LGKM0();
             const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP + (c_first >= 0 ? Cfg::C_PER_SLICE : 0);
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
-            constexpr int KMAX0 = 2 * (LA > LB ? LA : LB) * 3, KC3 = Cfg::C_PREFETCH ? 3 * Cfg::C_PER_SLICE : 0;
+            constexpr int KMAX0 = 2 * (LA > LB ? LA : LB) * 3, KC3 = OLD_C_AHEAD ? 3 * Cfg::C_PER_SLICE : 0;
             constexpr int KMAX = ((KMAX0 > KC3 ? KMAX0 : KC3) + G - 1) / G * G;
             bool waited = false;
             static_for<KMAX / G>([&](auto Q) {
@@ -849,7 +858,7 @@ gemm_x16_kernel(const GemmArgs args)
             // under the last four slices and is waiting in the ring buffers those slices left (c_ahead)
             u32x4 cold[FM * FN / 2];
             bool from_lds = false;
-            if constexpr (Cfg::C_PREFETCH && PAIR) {
+            if constexpr (OLD_C_AHEAD) {
                 if (c_ahead) {
                     from_lds = true;
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wavefront's own loads: nobody else reads them

@@ -250,6 +250,31 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
     assert ran >= 40 * 16
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (1, 1), (0, 1)])
+def test_x16_kernel_old_c_fetched_under_the_last_slices(ta, tb):
+    """fp16 with beta != 0: on whole tiles with at least ring-depth + 1 whole slices the x16 kernel fetches the tile's old C
+    into the LDS ring buffers its last four slices leave (a kernel variant of its own, for the layouts with paired loads:
+    NN, TN, TT; NT keeps reading C in the epilogue).  Slice counts on both sides of that limit and of either parity, every
+    tile that has the variant and the two that have not, several tiles per resident work-group, batches, ldc > m; the
+    reference's own epilogue order is t = alpha * acc, then fma(beta, C, t) (MT192x096x08 kernel :2300-2316, :3037-3056)."""
+    import gemm_mmbo_amd as G
+    ids = [c for c in _x16_ids(F16) if G.config_info(F16, c)["split_k"] == 1]
+    assert len(ids) == 8
+    ran = 0
+    for cid in ids:
+        d = G.config_info(F16, cid)
+        bm, bn = d["macro_tile_m"], d["macro_tile_n"]
+        depth = d["lds_bytes"] // ((bm + bn) * 64)
+        for slices in (depth, depth + 1, depth + 2, depth + 3, depth + 4, 2 * depth + 3):
+            tm, tn, batch = (3, 2, 1) if slices == depth + 2 else (1, 1, 2) if slices == depth + 3 else (1, 1, 1)
+            m, n, k = bm * tm, bn * tn, 32 * slices
+            p = U.Problem(F16, ta, tb, m, n, k, -0.75, 0.5, ldc=m + (8 if slices % 2 else 0), batch=batch, seed=500 + cid + slices,
+                          dist="normal", c_fill="uniform")
+            _run_and_check(p, cid, label=f"{d['name']} {'NT'[ta]}{'NT'[tb]} {m}x{n}x{k} b{batch}")
+            ran += 1
+    assert ran == 48
+
+
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
     ragged border of tiles, against the oracle.  Unaligned operands are taken, a contiguous dimension shorter than one

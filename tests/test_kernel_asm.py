@@ -82,7 +82,7 @@ def _inflight_violations(body):
 
     The walk follows one kind of infeasible path no further: for `if (c) A else B` between two long straight-line
     blocks the compiler emits "B (when !c), flag = 0 -- or flag = -1 -- then: A when flag", with the flag in a scalar
-    register pair (`s_mov_b64 s[a:b], 0` / `-1` ... `s_and_b64 vcc, exec, s[a:b]` ... `s_cbranch_vccz`).  The state
+    register pair (`s_mov_b64 s[a:b], 0` / `-1` ... `s_and_b64` or `s_andn2_b64 vcc, exec, s[a:b]` ... `s_cbranch_vccz` / `vccnz`).  The state
     therefore carries the flags whose constant value is known on the path at hand, and a branch on such a flag has one
     successor."""
     label = {t[:-1]: i for i, t in enumerate(body) if t.endswith(":")}
@@ -93,10 +93,11 @@ def _inflight_violations(body):
         if m:
             key = (int(m.group(1)), int(m.group(2)))
             return frozenset({f for f in flags if f[0] != key} | {(key, 0 if m.group(3) == "0" else 1)}), vcc
-        m = re.match(r"s_and_b64 vcc, exec, s\[(\d+):(\d+)\]$", t)
+        m = re.match(r"s_(and|andn2)_b64 vcc, exec, s\[(\d+):(\d+)\]$", t)
         if m:
-            key = (int(m.group(1)), int(m.group(2)))
-            return flags, next((v for k, v in flags if k == key), None)
+            key = (int(m.group(2)), int(m.group(3)))
+            known = next((v for k, v in flags if k == key), None)
+            return flags, known if known is None or m.group(1) == "and" else 1 - known
         if t.startswith(("s_", "v_cmp", "v_readlane", "v_readfirstlane")) and not t.startswith(("s_cbranch", "s_branch", "s_waitcnt", "s_nop", "s_barrier")):
             dst = t.split(None, 1)[1].split(",")[0] if " " in t else ""
             if "vcc" in dst or t.startswith("v_cmp"):
@@ -168,6 +169,10 @@ def test_checker_follows_a_constant_flag_but_not_an_unknown_one():
     assert _inflight_violations(overwritten) == ["v_add_u32_e32 v11, s3, v9"]
     set_one = ["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], -1", ".LBB0_8:"] + tail
     assert _inflight_violations(set_one) == ["v_add_u32_e32 v11, s3, v9"]
+    # the complemented form: vcc = exec & ~flag, skip A when vcc != 0
+    tail2 = ["s_andn2_b64 vcc, exec, s[6:7]", "s_cbranch_vccnz .LBB0_9"] + tail[2:]
+    assert _inflight_violations(["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], 0", ".LBB0_8:"] + tail2) == []
+    assert _inflight_violations(["ds_read_b128 v[10:13], v5 offset:64", "s_mov_b64 s[6:7], -1", ".LBB0_8:"] + tail2) == ["v_add_u32_e32 v11, s3, v9"]
 
 
 def test_checker_sees_a_planted_violation():
@@ -323,4 +328,4 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
-    assert seen == 64
+    assert seen == 82          # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 3 paired layouts with the old-C variant
