@@ -313,10 +313,13 @@ struct X16Cfg {
     static_assert(BATCH * (DEPTH - 1) < 64, "more loads in flight than vmcnt can count");
     // Old C ahead of the epilogue (fp16, beta != 0): a wavefront's FM * FN / 2 sixteen-byte groups per lane (two vertically
     // adjacent blocks each, as the epilogue reads them) are fetched with direct loads into the ring buffers the last
-    // slices no longer need, a quarter of them under each of the last four slices.
+    // slices no longer need, a quarter of them under each of the last four slices, evenly spread over the slice's MFMAs.
     static constexpr int C_GROUPS = FM * FN / 2;
-    static constexpr int C_PER_SLICE = C_GROUPS / 4;
-    static constexpr bool C_PREFETCH = ESZ == 2 && FM % 2 == 0 && C_GROUPS % 4 == 0 && C_PER_SLICE * 8 == NMFMA &&
+    static constexpr int C_PER_SLICE = (C_GROUPS + 3) / 4;                       // (the last of the four slices may carry fewer)
+    static constexpr int C_PERIOD = NMFMA / (C_PER_SLICE > 0 ? C_PER_SLICE : 1);  // one load every C_PERIOD MFMAs
+    // (wave tiles of 64 x 64 and more: on the 64 x 64 macro tile the variant's longer tails cost more than the read it hides,
+    // HGEMM 1000 x 1000 x 1024 with beta = 1: 9.5 -> 9.7 us)
+    static constexpr bool C_PREFETCH = ESZ == 2 && FM % 2 == 0 && C_GROUPS >= 8 && C_PERIOD >= 2 &&
                                        C_PER_SLICE * NW * 1024 <= SLICE_BYTES;
 };
 
@@ -551,11 +554,13 @@ gemm_x16_kernel(const GemmArgs args)
                     if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b, DESTINATION_SET);
                 }
             });
-            if constexpr (old_c && OLD_C_AHEAD && m % 8 == 3) {
-                constexpr int c = m / 8;
+            if constexpr (old_c && OLD_C_AHEAD && m % Cfg::C_PERIOD == Cfg::C_PERIOD / 2 && m / Cfg::C_PERIOD < Cfg::C_PER_SLICE) {
+                constexpr int c = m / Cfg::C_PERIOD;
                 const uint32_t q = (uint32_t)c_first + c;             // group q: column block q / (FM / 2), row-block pair q % (FM / 2)
-                const uint32_t soff = __builtin_amdgcn_readfirstlane((q / (FM / 2)) * c_col_step + (q % (FM / 2)) * (32 * ESZ));
-                direct_load16<true>(curC, soff, c_lane_off, c_dst + c * 1024);
+                if (Cfg::C_GROUPS % Cfg::C_PER_SLICE == 0 || q < (uint32_t)Cfg::C_GROUPS) {
+                    const uint32_t soff = __builtin_amdgcn_readfirstlane((q / (FM / 2)) * c_col_step + (q % (FM / 2)) * (32 * ESZ));
+                    direct_load16<true>(curC, soff, c_lane_off, c_dst + c * 1024);
+                }
             }
             // (one scheduling barrier per MFMA slot, at its end: two of them with nothing in between make the compiler
             // pad the gap with an s_nop, which costs an issue slot like any other instruction)
@@ -690,7 +695,8 @@ gemm_x16_kernel(const GemmArgs args)
             }
             advance_op(std::integral_constant<int, par ^ EVEN_OP>{}, 2);
             MMBO_WAIT_LGKM0();
-            const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP + (c_first >= 0 ? Cfg::C_PER_SLICE : 0);
+            const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP +
+                            (c_first >= 0 ? max(0, min(Cfg::C_PER_SLICE, Cfg::C_GROUPS - c_first)) : 0);
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
             constexpr int KMAX0 = 2 * (LA > LB ? LA : LB) * 3, KC3 = OLD_C_AHEAD ? 3 * Cfg::C_PER_SLICE : 0;
             constexpr int KMAX = ((KMAX0 > KC3 ? KMAX0 : KC3) + G - 1) / G * G;
@@ -871,7 +877,7 @@ gemm_x16_kernel(const GemmArgs args)
                         const uint32_t at = mine + b * Cfg::SLICE_BYTES;
                         static_for<Cfg::C_PER_SLICE>([&](auto Q) {
                             constexpr int q = decltype(Q)::value;
-                            cold[cc * Cfg::C_PER_SLICE + q] = lds_read_b128<q * 1024>(at);
+                            if constexpr (cc * Cfg::C_PER_SLICE + q < Cfg::C_GROUPS) cold[cc * Cfg::C_PER_SLICE + q] = lds_read_b128<q * 1024>(at);
                         });
                     });
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
