@@ -328,14 +328,14 @@ struct X16Cfg {
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
 // one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
 // OLD_C_AHEAD: the variant for beta != 0 that fetches a tile's old C into LDS under the tile's last four slices (see c_ahead
-// below).  A kernel of its own, chosen by the host: with the code in the one kernel, calls that have no C to read paid
+// below; both load schedules).  A kernel of its own, chosen by the host: with the code in the one kernel, calls that have no C to read paid
 // 1.5-3 % on short-k and mid-size shapes for tails that had grown.
 template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, bool PAIR = (TA || !TB),
           int EVEN_OP = (TA ? 0 : 1), bool OLD_C_AHEAD = false>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_x16_kernel(const GemmArgs args)
 {
-    static_assert(!OLD_C_AHEAD || (PAIR && X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>::C_PREFETCH), "no old-C variant of this kernel");
+    static_assert(!OLD_C_AHEAD || X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>::C_PREFETCH, "no old-C variant of this kernel");
     using namespace x16;
     using Cfg = X16Cfg<T, TA, TB, BM, BN, WM, WN, DEPTH>;
     using TileA = typename Cfg::TileA;
@@ -618,6 +618,22 @@ gemm_x16_kernel(const GemmArgs args)
         auto tail_step = [&](int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             const bool load = s + DEPTH < n_slice;
+            if constexpr (OLD_C_AHEAD) {
+                // The last four slices carry the old C (no operand load is issued in the last DEPTH slices).  All operand loads
+                // are older than any of these; loads return in order, so leaving at most two slices' worth of C loads in flight
+                // also means every operand load has landed -- except, under the first of the four slices, some of the newest
+                // C_PER_SLICE operand loads, which belong to the last slice (C_PER_SLICE <= BATCH) and are not needed yet.
+                static_assert(Cfg::C_PER_SLICE <= BATCH && 2 * Cfg::C_PER_SLICE < 64, "old-C loads per slice exceed what the wait below assumes");
+                const int c_first = __builtin_amdgcn_readfirstlane((c_ahead && s + 4 >= n_slice) ? (s + 4 - n_slice) * Cfg::C_PER_SLICE : -1);
+                if (c_first >= 0) {
+                    mfma_and_read(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, false, false, buf, std::true_type{}, c_first);
+                    MMBO_WAIT_LGKM0();
+                    MMBO_WAIT_VM(2 * Cfg::C_PER_SLICE);
+                    MMBO_BARRIER();
+                    buf = nbuf;
+                    return;
+                }
+            }
             mfma_and_read(std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{}, ca, cb, na, nb, nbuf, load, load, buf, std::false_type{}, 0);
             MMBO_WAIT_LGKM0();
             if (load) MMBO_WAIT_VM(BATCH * (DEPTH - 2)); else MMBO_WAIT_VM(0);

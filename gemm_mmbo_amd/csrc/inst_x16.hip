@@ -21,7 +21,7 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
     using Cfg = X16Cfg<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
     // beta != 0 on fp16 (args.c_prefetch): the variant that fetches the old C ahead of the epilogue, where the tile has one
-    if constexpr (!OLD_C && Cfg::C_PREFETCH && (TA || !TB)) {
+    if constexpr (!OLD_C && Cfg::C_PREFETCH) {
         if (args.c_prefetch) return launch_one<TA, TB, WM, WN, true>(args, stream);
     }
     auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth, (TA || !TB), (TA ? 0 : 1), OLD_C>;

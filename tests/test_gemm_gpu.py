@@ -253,8 +253,8 @@ def test_x16_kernel_edge_tiles_and_partial_last_slice(dtype, ta, tb):
 @pytest.mark.parametrize("ta,tb", [(0, 0), (1, 0), (1, 1), (0, 1)])
 def test_x16_kernel_old_c_fetched_under_the_last_slices(ta, tb):
     """fp16 with beta != 0: on whole tiles with at least ring-depth + 1 whole slices the x16 kernel fetches the tile's old C
-    into the LDS ring buffers its last four slices leave (a kernel variant of its own, for the layouts with paired loads:
-    NN, TN, TT; NT keeps reading C in the epilogue).  Slice counts on both sides of that limit and of either parity, every
+    into the LDS ring buffers its last four slices leave (a kernel variant of its own, in both load schedules: the paired one
+    of NN, TN, TT and the plain one of NT).  Slice counts on both sides of that limit and of either parity, every
     tile (those of 128 x 128 and more have the variant; the 192 x 192 one carries fewer groups under the last of the four slices), several tiles per resident work-group, batches, ldc > m; the
     reference's own epilogue order is t = alpha * acc, then fma(beta, C, t) (MT192x096x08 kernel :2300-2316, :3037-3056)."""
     import gemm_mmbo_amd as G

@@ -328,4 +328,4 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
-    assert seen == 82          # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 3 paired layouts with the old-C variant
+    assert seen == 88          # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 4 transposes with the old-C variant
