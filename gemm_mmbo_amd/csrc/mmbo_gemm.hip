@@ -509,8 +509,12 @@ static double model_time_tile(int dtype, const RingRow &r, double e, int split, 
         // A last round that leaves CUs idle runs faster per tile on fp16: the chip is power-limited on these MFMAs and the
         // clock rises when fewer CUs draw power (HGEMM 3072^3 on 144 tiles of 256 x 256: 54 us against 74 us for a full
         // round of the same tiles; 5120^3, 256 + 144 tiles: the second round takes 0.82 of the first).
-        const double busy = last >= cus ? 1.0 : last / cus;
-        const double boost = dtype == MMBO_F16 ? 0.45 + 0.55 * busy : 1.0;
+        // (with several work-groups to a CU the round lasts as long as the fullest CU's; "busy" is the share of CU time in use)
+        const double busy = last / (cus * std::ceil(last / cus));
+        // (the tiles that run one to a CU are the power-limited ones; the smaller ones, bound by the L2 -> LDS stream, gain
+        // less: HGEMM 1280 x 1280 x 4096 on 100 tiles of 128 x 128 runs at 0.86 of a full round's time per tile)
+        const bool one_per_cu = r.depth * (r.bm + r.bn) * 64 > 80 * 1024;
+        const double boost = dtype != MMBO_F16 ? 1.0 : one_per_cu ? 0.45 + 0.55 * busy : 0.7 + 0.3 * busy;
         t += tile_time(std::ceil(last / cus)) * boost;
     }
     if (split > 1) t += reduce_launch + reduce_us_per_mb * (double)m * n * batch * (split * 4.0 + esz) / 1e6;
