@@ -118,7 +118,8 @@ int mmbo_select_config(int dtype, int transA, int transB, size_t m, size_t n, si
 int mmbo_wg_remap(unsigned linear_id, unsigned nwg0, unsigned nwg1, unsigned wgm, unsigned num_xcd,
                   unsigned *wg0, unsigned *wg1);
 
-/* Host twin of the order in which the 256 x 256 HGEMM tiles are walked on grids of at least 16 x 16 tiles: chip-wide
+/* Host twin of the order in which the tiles that run one work-group per CU (256 x 256, 192 x 192, 256 x 192, 192 x 256 of
+ * the 16x16-block kernel) are walked on grids of at least 16 x 16 tiles: chip-wide
  * blocks of 16 x 16 tiles (one per CU at a time), each XCD (linear_id % 8) on a 4 x 8 sub-block, blocks in
  * serpentine order, so the operand panels in flight at one time fit the last-level cache.  The reference maps
  * work-groups for its one L2 only (src/gemm/ref/Kernels.cpp:204-236); this is that idea one cache level up.
