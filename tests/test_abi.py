@@ -244,3 +244,24 @@ def test_ragged_shapes_go_to_the_fast_kernels():
     assert "DTL1" in name(G.F16, 0, 0, 72, 4096, 4096)
     # large ragged shapes whose packed rows split cache lines: the 256 x 256 tile, not the bandwidth-bound smaller ones
     assert G.config_info(G.F16, G.select_config(G.F16, 1, 0, 7000, 7000, 7008))["macro_tile_m"] == 256
+
+
+def test_sizes_between_rounds_of_the_cus_get_the_192_tiles():
+    """3000^2 is 144 tiles of 256 x 256 -- little more than half of the 256 CUs -- but 256 tiles of 192 x 192; the pick
+    follows the tile counts (the reference keeps such knowledge in its exact-size table,
+    src/gemm/ref/vega20_Cijk_Ailk_Bjlk_DB.yaml:929-1177).  Sizes that fill whole rounds keep the 256 x 256 tile."""
+    def tile(dtype, m, n, k, ta=0, tb=0):
+        d = G.config_info(dtype, G.select_config(dtype, ta, tb, m, n, k))
+        return d["macro_tile_m"], d["macro_tile_n"]
+    assert tile(G.F16, 3000, 3000, 3000) == (192, 192) and tile(G.F16, 3072, 3072, 3072) == (192, 192)
+    assert tile(G.F32, 3072, 3072, 3072) == (192, 192)
+    assert tile(G.F16, 3328, 3328, 3328) in ((256, 192), (192, 256)) and tile(G.F16, 4608, 4608, 4608) in ((256, 192), (192, 256))
+    for s in (3584, 4096, 5120, 8192):
+        assert tile(G.F16, s, s, s) == (256, 256), s
+    assert tile(G.F16, 2048, 2048, 2048) == (128, 128) and tile(G.F16, 2560, 2560, 2560) == (128, 128)
+    # the three tiles exist for both element types and every GlobalSplitU, one work-group per CU (more than 80 KB of LDS)
+    for dtype in (G.F16, G.F32):
+        big = [G.config_info(dtype, c) for c in range(G.num_configs(dtype))]
+        for mt in ((192, 192), (256, 192), (192, 256)):
+            rows = [d for d in big if (d["macro_tile_m"], d["macro_tile_n"]) == mt]
+            assert sorted(d["split_k"] for d in rows) == [1, 2, 4, 8, 16] and all(d["lds_bytes"] > 80 * 1024 and d["threads"] == 256 for d in rows)
