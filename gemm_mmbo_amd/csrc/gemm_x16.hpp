@@ -865,10 +865,22 @@ gemm_x16_kernel(const GemmArgs args)
     // Two results at a time go through the packed conversion (round to nearest even, like the scalar cast).
     constexpr bool PAIRED_C = ESZ == 2 && FM % 2 == 0;
     const uint32_t pair_row0 = row0 + wm * Cfg::TM + (((lane >> 4) & 1) ? 4 * (lane >> 4) + 12 : 4 * (lane >> 4));
-    // C goes out with the non-temporal hint: the kernel never reads what it wrote, and a resident work-group's 128 KB per
-    // tile (4 MB per XCD and round of tiles: the size of its L2) otherwise push the operand panels the next tiles share out
-    // of the L2 (measured at 8192^3 fp16: the epilogue itself takes 1 us longer, the next tile's loop 3-6 us less).
-    auto store_c = [](auto value, auto *where) { __builtin_nontemporal_store(value, where); };
+    // C leaves with the non-temporal hint where the host asks for it (args.c_stream: a long slice loop and several rounds of
+    // tiles per CU): the kernel never reads what it wrote, and a resident work-group's 128 KB per tile (4 MB per XCD and round
+    // of tiles: the size of its L2) otherwise push the operand panels the next tiles share out of the L2 (measured at 8192^3
+    // fp16: the epilogue itself takes 1 us longer, the next tile's loop 3-6 us less).  Everywhere else plain stores: with
+    // the hint the two 64-byte halves of a line travel to memory separately, and where the epilogue is on the critical path
+    // (one round of tiles, short k) that is what the kernel then waits for (64 x 512^3 fp16: 7.4 us to issue a
+    // wavefront's 32 stores against 3.5).  One copy of each store sequence per policy, chosen once.
+    const bool c_stream = args.c_stream != 0;
+    auto store_c = [](auto STREAM, auto value, auto *where) {
+        if constexpr (decltype(STREAM)::value) __builtin_nontemporal_store(value, where);
+        else *where = value;
+    };
+    auto per_policy = [&](auto &&body) {
+        if (c_stream) body(std::true_type{});
+        else body(std::false_type{});
+    };
     auto two = [](float a, float b) -> uint32_t {
         typedef float f32x2 __attribute__((ext_vector_type(2)));
         typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -907,6 +919,7 @@ gemm_x16_kernel(const GemmArgs args)
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
                 cold[decltype(IJ)::value] = *reinterpret_cast<const u32x4 *>(C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16);
             });
+            per_policy([&](auto STREAM) {
             static_for<FM * FN / 2>([&](auto IJ) {
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
                 constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
@@ -926,7 +939,8 @@ gemm_x16_kernel(const GemmArgs args)
                 auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
                 auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
                 T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
-                store_c(u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
+                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
+            });
             });
             continue;
         }
@@ -934,6 +948,7 @@ gemm_x16_kernel(const GemmArgs args)
         // old C (fp16: the whole wave tile) is requested before its first value is used, so the read-modify-write runs
         // at memory bandwidth instead of one load latency per block.
         constexpr int CHUNK = ESZ == 2 ? FM * FN : FM;                          // blocks requested at once
+        per_policy([&](auto STREAM) {
         static_for<FM * FN / CHUNK>([&](auto CC) {
             constexpr int c0 = decltype(CC)::value * CHUNK;
             cvec cold[CHUNK];
@@ -949,8 +964,9 @@ gemm_x16_kernel(const GemmArgs args)
                 float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
 #pragma unroll
                 for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], v[r]);
-                store_c(io.v, reinterpret_cast<cvec *>(p));
+                store_c(STREAM, io.v, reinterpret_cast<cvec *>(p));
             });
+        });
         });
         continue;
     }
@@ -960,7 +976,7 @@ gemm_x16_kernel(const GemmArgs args)
     if (vec_c && PAIRED_C) {
         // alpha == 1 gets a copy of the sequence without the multiplications: with the packed conversions that makes 4 (12)
         // instructions per eight results where scalar casts took 16.
-        auto store_all = [&](auto UNIT_ALPHA) {
+        auto store_all = [&](auto UNIT_ALPHA, auto STREAM) {
             constexpr bool unit = decltype(UNIT_ALPHA)::value;
             static_for<FM * FN / 2>([&](auto IJ) {
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
@@ -974,12 +990,15 @@ gemm_x16_kernel(const GemmArgs args)
                 auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
                 auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
                 T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
-                store_c(u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
+                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
             });
         };
-        if (alpha == 1.0f) store_all(std::true_type{});
-        else store_all(std::false_type{});
+        per_policy([&](auto STREAM) {
+            if (alpha == 1.0f) store_all(std::true_type{}, STREAM);
+            else store_all(std::false_type{}, STREAM);
+        });
     } else if (vec_c) {
+        per_policy([&](auto STREAM) {
         static_for<FM * FN>([&](auto IJ) {
             constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
             T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
@@ -988,7 +1007,8 @@ gemm_x16_kernel(const GemmArgs args)
             io.e[1] = (T)(alpha * acc_read<base + 1>());
             io.e[2] = (T)(alpha * acc_read<base + 2>());
             io.e[3] = (T)(alpha * acc_read<base + 3>());
-            store_c(io.v, reinterpret_cast<cvec *>(p));
+            store_c(STREAM, io.v, reinterpret_cast<cvec *>(p));
+        });
         });
     } else {
         static_for<FM * FN>([&](auto IJ) {

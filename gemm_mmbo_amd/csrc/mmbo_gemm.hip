@@ -822,6 +822,10 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
     // tile's span of C, tile columns x ldc, must then fit the 32-bit offsets of a buffer load)
     a.c_prefetch = cref.x16 && dtype == MMBO_F16 && beta_f != 0.0f && split == 1 && a.vec_c &&
                    (size_t)r.bn * ldc * esz < 0x7FFFFF00ull;
+    // C with the non-temporal hint: only where resident work-groups walk at least four rounds of tiles (256 CUs) with a long
+    // slice loop -- there the operand panels the next tiles share are worth more in the L2 than a fast epilogue (8192^3:
+    // +0.3 %); with fewer rounds or a short k plain stores win (fp16 6144^3 +1.6 %, 44160 x 2048 x 384 +2.7 %, 64 x 512^3 +14 %)
+    a.c_stream = cref.x16 && rr.depth * (rr.bm + rr.bn) * 64 > 80 * 1024 && (size_t)nwg0 * nwg1 >= 4 * 256 && k >= 4096;
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (cref.ring && !cref.x16 && (!a.vec_a || !a.vec_b)) return MMBO_ERR_INVALID_CONFIG;
