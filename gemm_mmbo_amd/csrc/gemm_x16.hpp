@@ -654,26 +654,46 @@ gemm_x16_kernel(const GemmArgs args)
         constexpr int LA = EVEN_OP == 0 ? TileA::LPW : TileB::LPW, LB = EVEN_OP == 0 ? TileB::LPW : TileA::LPW;
         constexpr std::integral_constant<int, EVEN_OP> OPX{};
         constexpr std::integral_constant<int, 1 - EVEN_OP> OPY{};
-        // prologue: X slices 0 .. DEPTH-2, Y slices 0 .. DEPTH-1, slice by slice (iteration 0 brings X's DEPTH-1 and DEPTH)
-#pragma unroll
-        for (int q = 0; q < DEPTH; ++q) {
-            if (q < n_slice) {
-                if (q < DEPTH - 1) {
-                    static_for<LA>([&](auto I) { issue_op_load(OPX, I, std::false_type{}, op_dst(OPX, q), std::false_type{}); });
-                    advance_op(OPX, 1);
-                }
-                static_for<LB>([&](auto I) { issue_op_load(OPY, I, std::false_type{}, op_dst(OPY, q), std::false_type{}); });
-                advance_op(OPY, 1);
+        // prologue: X slices 0 .. DEPTH-2, Y slices 0 .. DEPTH-1 (iteration 0 brings X's DEPTH-1 and DEPTH).  Slices 0 and 1 of both
+        // operands -- and, with five buffers, X's 2 and 3 -- go out the way the loop's pairs do, the two loads that share a memory
+        // line back to back (whole-line requests stream twice as fast as half-line ones, and nothing else is in flight yet);
+        // the rest slice by slice, in the order the loop's first waits count on: they let the newest loads of the prologue stay
+        // in flight, and none of those may belong to slice 2.
+        auto pro_pair = [&](auto OP, auto L, int q) {                    // slices q and q + 1 of one operand
+            constexpr int n = decltype(L)::value;
+            if (q + 1 < n_slice) {
+                static_for<n>([&](auto I) {
+                    issue_op_load(OP, I, std::false_type{}, op_dst(OP, q), std::false_type{});
+                    issue_op_load(OP, I, std::true_type{}, op_dst(OP, q + 1), std::false_type{});
+                });
+            } else if (q < n_slice) {
+                static_for<n>([&](auto I) { issue_op_load(OP, I, std::false_type{}, op_dst(OP, q), std::false_type{}); });
             }
+            advance_op(OP, 2);                                           // (not under the branch: the cursors stay in scalar registers)
+        };
+        auto pro_one = [&](auto OP, auto L, int q) {
+            constexpr int n = decltype(L)::value;
+            if (q < n_slice) static_for<n>([&](auto I) { issue_op_load(OP, I, std::false_type{}, op_dst(OP, q), std::false_type{}); });
+            advance_op(OP, 1);
+        };
+        constexpr std::integral_constant<int, LA> NLA{};
+        constexpr std::integral_constant<int, LB> NLB{};
+        constexpr int X_PAIRED = DEPTH == 5 ? 4 : 2;                     // X's slices below this go out in pairs
+        pro_pair(OPX, NLA, 0);
+        pro_pair(OPY, NLB, 0);
+        if constexpr (X_PAIRED == 4) pro_pair(OPX, NLA, 2);
+#pragma unroll
+        for (int q = 2; q < DEPTH; ++q) {
+            if (q >= X_PAIRED && q < DEPTH - 1) pro_one(OPX, NLA, q);
+            pro_one(OPY, NLB, q);
         }
         constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
         acc_zero<NACC>();                                                // (while the first slices are on their way)
-        if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - BATCH); else MMBO_WAIT_VM(0);
-        MMBO_BARRIER();                                                  // slice 0 resident
+        if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - 2 * BATCH); else MMBO_WAIT_VM(0);
+        MMBO_BARRIER();                                                  // slices 0 and 1 resident
         read_slice(fa[0], fb[0], 0);
         MMBO_WAIT_LGKM0();
-        if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - 2 * BATCH); else MMBO_WAIT_VM(0);
-        MMBO_BARRIER();                                                  // slice 1 resident, slice 0 in registers
+        MMBO_BARRIER();                                                  // slice 0 in registers
 
         // loads a steady iteration of parity P leaves in flight: those of the last DEPTH-3 iterations, itself included
         auto steady_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
