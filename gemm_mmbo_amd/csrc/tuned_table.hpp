@@ -35,7 +35,7 @@ constexpr TunedRow kTuned[] = {
     {1, 0, 0, 4096, 128, 4096, 1, ring_id(3, 2), 276.1f},
     {0, 0, 0, 128, 4096, 8192, 1, ring_id(1, 8), 118.9f},
     {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 425.8f},
-    {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 567.0f},
+    {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 650.0f},
     {0, 0, 0, 2048, 2048, 2048, 1, x16_id(3, 1), 132.6f},
     {1, 0, 0, 2048, 2048, 2048, 1, x16_id(2, 1), 834.2f},
     {0, 0, 1, 44160, 2048, 384, 1, ring_id(1, 1), 128.0f},
