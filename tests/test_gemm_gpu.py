@@ -461,6 +461,30 @@ def test_identity_and_ones_closed_forms_full_size(dtype, size):
 
 
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_old_c_closed_form_where_c_leaves_with_the_streaming_hint(dtype):
+    """8192 x 8192 x 4096 on the 256 x 256 tile is 1,024 tiles with k >= 4096: the shape class whose C is stored with the
+    non-temporal hint.  With beta != 0 and alpha != 1 on all-ones operands every result is 0.25*K + 0.5*C0, exact for
+    small even integers in C0 -- a bitwise check of that store sequence (and of the old C fetched ahead of it) without an
+    oracle run; the plain-store copies of the same sequences are what every smaller test exercises."""
+    import torch
+    import gemm_mmbo_amd as G
+    tdt = torch.float32 if dtype == F32 else torch.float16
+    m = n = 8192
+    k = 4096
+    cid = G.select_config(dtype, 0, 0, m, n, k)
+    assert "MT256x256" in G.config_info(dtype, cid)["name"]
+    ones_a = torch.ones(m * k, dtype=tdt, device="cuda")
+    ones_b = torch.ones(k * n, dtype=tdt, device="cuda")
+    C0 = (torch.arange(m * n, device="cuda", dtype=torch.int64) % 32 * 2).to(tdt)
+    want = 0.25 * k + 0.5 * C0
+    for (ta, tb) in ((0, 0), (0, 1)):
+        C = C0.clone()
+        G.gemm(dtype, ta, tb, m, n, k, 0.25, ones_a, m if not ta else k, ones_b, k if not tb else n, 0.5, C, m)
+        torch.cuda.synchronize()
+        assert torch.equal(C, want), (ta, tb)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_linearity_in_alpha_and_beta(dtype):
     """gemm(2a, 2b) == 2 * gemm(a, b) bit for bit: scaling by two is exact in binary floating point
     (outside the fp16 subnormal range, where the doubled value has one more significant bit to round)."""
