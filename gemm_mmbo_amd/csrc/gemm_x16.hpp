@@ -885,17 +885,38 @@ gemm_x16_kernel(const GemmArgs args)
     // Two results at a time go through the packed conversion (round to nearest even, like the scalar cast).
     constexpr bool PAIRED_C = ESZ == 2 && FM % 2 == 0;
     const uint32_t pair_row0 = row0 + wm * Cfg::TM + (((lane >> 4) & 1) ? 4 * (lane >> 4) + 12 : 4 * (lane >> 4));
-    // C leaves with the non-temporal hint where the host asks for it (args.c_stream: a long slice loop and several rounds of
-    // tiles per CU): the kernel never reads what it wrote, and a resident work-group's 128 KB per tile (4 MB per XCD and round
-    // of tiles: the size of its L2) otherwise push the operand panels the next tiles share out of the L2 (measured at 8192^3
-    // fp16: the epilogue itself takes 1 us longer, the next tile's loop 3-6 us less).  Everywhere else plain stores: with
-    // the hint the two 64-byte halves of a line travel to memory separately, and where the epilogue is on the critical path
-    // (one round of tiles, short k) that is what the kernel then waits for (64 x 512^3 fp16: 7.4 us to issue a
-    // wavefront's 32 stores against 3.5).  One copy of each store sequence per policy, chosen once.
+    // The whole-tile store sequences below address C as a buffer whose origin is the tile's first element (the host lets
+    // vec_c stand only where a tile's span of C, BN x ldc elements, fits the 32-bit offsets of a buffer access): the lane's
+    // part of an address is worked out once, a block adds its column (one vector addition per block column) and, as an
+    // immediate, its row.  (The column as the instruction's scalar offset would save that addition, but the compiler then
+    // leaves out the wait states between a 16-byte store and the next write to its data registers -- it takes them to be
+    // needed only without a scalar offset -- and with the accumulator reads of the next block right behind the store
+    // a few lanes stored the next block's value: seen on the 8-wave fp32 tile.)
+    // Two cache policies, one copy of each store sequence per policy, chosen once:
+    // * device scope (sc1) by default: the stores go through the XCD's L2 to memory as they are made.  Left in the L2 as
+    //   ordinary stores are, C is written back when the kernel ends, and where the epilogue is on the critical path (one
+    //   round of tiles, short k) that is time added at the end: 64 x 512^3 fp16 26.6 -> 25.7 us, 2048^3 21.6 -> 20.9;
+    // * non-temporal where the host asks for it (args.c_stream: a long slice loop and four or more rounds of tiles per CU):
+    //   the kernel never reads what it wrote, and a resident work-group's 128 KB per tile (4 MB per XCD and round of tiles:
+    //   the size of its L2) otherwise push the operand panels the next tiles share out of the L2 (measured at 8192^3 fp16:
+    //   the epilogue itself takes 1 us longer, the next tile's loop 3-6 us less).  Not everywhere: with this hint the two
+    //   64-byte halves of a line travel to memory separately (64 x 512^3 fp16: 7.4 us to issue a wavefront's 32 stores
+    //   against 3.5).
     const bool c_stream = args.c_stream != 0;
-    auto store_c = [](auto STREAM, auto value, auto *where) {
-        if constexpr (decltype(STREAM)::value) __builtin_nontemporal_store(value, where);
-        else *where = value;
+    const T *c_origin = C + (size_t)col0 * ldc + row0;
+    // (the descriptor is put together inside each copy, from an address that has just passed through readfirstlane: built once
+    // up here it reached some of the copies in vector registers, and every store became a loop over the distinct descriptors)
+    auto c_buffer = [&]() {
+        return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(uniform_address(c_origin)), 0, 0x7fffffff, 0x00020000);
+    };
+    const uint32_t c_block_col = 16 * ldc * ESZ;                          // bytes from a block's column to the next block's
+    // this lane's first element of the wave tile: four rows of one column per block, or, fp16 pairs, eight rows of two blocks
+    const uint32_t c_lane = ((wn * Cfg::TN + (lane & 15)) * ldc + wm * Cfg::TM + 4 * (lane >> 4)) * ESZ;
+    const uint32_t c_lane_pair = ((wn * Cfg::TN + (lane & 15)) * ldc + (pair_row0 - row0)) * ESZ;
+    auto store_c = [](auto STREAM, auto value, __amdgpu_buffer_rsrc_t tile_c, uint32_t lane_and_row, uint32_t column) {
+        constexpr int policy = decltype(STREAM)::value ? 2 : 16;            // nt : sc1
+        if constexpr (sizeof(value) == 16) __builtin_amdgcn_raw_buffer_store_b128(value, tile_c, lane_and_row, column, policy);
+        else __builtin_amdgcn_raw_buffer_store_b64(value, tile_c, lane_and_row, column, policy);
     };
     auto per_policy = [&](auto &&body) {
         if (c_stream) body(std::true_type{});
@@ -940,6 +961,7 @@ gemm_x16_kernel(const GemmArgs args)
                 cold[decltype(IJ)::value] = *reinterpret_cast<const u32x4 *>(C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16);
             });
             per_policy([&](auto STREAM) {
+            const __amdgpu_buffer_rsrc_t tile_c = c_buffer();
             static_for<FM * FN / 2>([&](auto IJ) {
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
                 constexpr int b0 = (i * FN + j) * 4, b1 = ((i + 1) * FN + j) * 4;
@@ -958,8 +980,7 @@ gemm_x16_kernel(const GemmArgs args)
                 }
                 auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
                 auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
-                T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
-                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
+                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, tile_c, c_lane_pair + j * c_block_col + i * 16 * ESZ, 0u);
             });
             });
             continue;
@@ -969,6 +990,7 @@ gemm_x16_kernel(const GemmArgs args)
         // at memory bandwidth instead of one load latency per block.
         constexpr int CHUNK = ESZ == 2 ? FM * FN : FM;                          // blocks requested at once
         per_policy([&](auto STREAM) {
+            const __amdgpu_buffer_rsrc_t tile_c = c_buffer();
         static_for<FM * FN / CHUNK>([&](auto CC) {
             constexpr int c0 = decltype(CC)::value * CHUNK;
             cvec cold[CHUNK];
@@ -978,13 +1000,12 @@ gemm_x16_kernel(const GemmArgs args)
             });
             static_for<CHUNK>([&](auto Q) {
                 constexpr int ij = c0 + decltype(Q)::value, j = ij / FM, i = ij % FM, base = (i * FN + j) * 4;
-                T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
                 union { T e[4]; cvec v; } io;
                 io.v = cold[decltype(Q)::value];
                 float v[4] = {alpha * acc_read<base>(), alpha * acc_read<base + 1>(), alpha * acc_read<base + 2>(), alpha * acc_read<base + 3>()};
 #pragma unroll
                 for (int r = 0; r < 4; ++r) io.e[r] = (T)__builtin_fmaf(beta, (float)io.e[r], v[r]);
-                store_c(STREAM, io.v, reinterpret_cast<cvec *>(p));
+                store_c(STREAM, io.v, tile_c, c_lane + j * c_block_col + i * 16 * ESZ, 0u);
             });
         });
         });
@@ -996,7 +1017,7 @@ gemm_x16_kernel(const GemmArgs args)
     if (vec_c && PAIRED_C) {
         // alpha == 1 gets a copy of the sequence without the multiplications: with the packed conversions that makes 4 (12)
         // instructions per eight results where scalar casts took 16.
-        auto store_all = [&](auto UNIT_ALPHA, auto STREAM) {
+        auto store_all = [&](auto UNIT_ALPHA, auto STREAM, __amdgpu_buffer_rsrc_t tile_c) {
             constexpr bool unit = decltype(UNIT_ALPHA)::value;
             static_for<FM * FN / 2>([&](auto IJ) {
                 constexpr int j = decltype(IJ)::value / (FM / 2), i = 2 * (decltype(IJ)::value % (FM / 2));
@@ -1009,25 +1030,25 @@ gemm_x16_kernel(const GemmArgs args)
                 }
                 auto s0 = __builtin_amdgcn_permlane16_swap(two(x[0], x[1]), two(y[0], y[1]), false, false);
                 auto s1 = __builtin_amdgcn_permlane16_swap(two(x[2], x[3]), two(y[2], y[3]), false, false);
-                T *p = C + (size_t)(wcol0 + j * 16) * ldc + pair_row0 + i * 16;
-                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, reinterpret_cast<u32x4 *>(p));
+                store_c(STREAM, u32x4{(uint32_t)s0[0], (uint32_t)s1[0], (uint32_t)s0[1], (uint32_t)s1[1]}, tile_c, c_lane_pair + j * c_block_col + i * 16 * ESZ, 0u);
             });
         };
         per_policy([&](auto STREAM) {
-            if (alpha == 1.0f) store_all(std::true_type{}, STREAM);
-            else store_all(std::false_type{}, STREAM);
+            const __amdgpu_buffer_rsrc_t tile_c = c_buffer();
+            if (alpha == 1.0f) store_all(std::true_type{}, STREAM, tile_c);
+            else store_all(std::false_type{}, STREAM, tile_c);
         });
     } else if (vec_c) {
         per_policy([&](auto STREAM) {
+            const __amdgpu_buffer_rsrc_t tile_c = c_buffer();
         static_for<FM * FN>([&](auto IJ) {
             constexpr int j = decltype(IJ)::value / FM, i = decltype(IJ)::value % FM, base = (i * FN + j) * 4;
-            T *p = C + (size_t)(wcol0 + j * 16) * ldc + wrow0 + i * 16;
             union { T e[4]; cvec v; } io;
             io.e[0] = (T)(alpha * acc_read<base>());
             io.e[1] = (T)(alpha * acc_read<base + 1>());
             io.e[2] = (T)(alpha * acc_read<base + 2>());
             io.e[3] = (T)(alpha * acc_read<base + 3>());
-            store_c(STREAM, io.v, reinterpret_cast<cvec *>(p));
+            store_c(STREAM, io.v, tile_c, c_lane + j * c_block_col + i * 16 * ESZ, 0u);
         });
         });
     } else {

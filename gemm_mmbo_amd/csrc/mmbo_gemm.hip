@@ -817,7 +817,9 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
     };
     a.vec_a = aligned16(A, lda, strideA);
     a.vec_b = aligned16(B, ldb, strideB);
-    a.vec_c = aligned16(C, ldc, strideC);
+    // (the x16 kernel's whole-tile epilogue addresses C as a buffer with 32-bit offsets: where a tile's span of C, its columns x
+    // ldc, does not fit them, C goes out element by element instead)
+    a.vec_c = aligned16(C, ldc, strideC) && (!cref.x16 || (size_t)r.bn * ldc * esz < 0x7FFFFF00ull);
     // beta != 0 on the x16 kernel's fp16 path: the old C of a tile is fetched into LDS under the tile's last slices (one
     // tile's span of C, tile columns x ldc, must then fit the 32-bit offsets of a buffer load)
     a.c_prefetch = cref.x16 && dtype == MMBO_F16 && beta_f != 0.0f && split == 1 && a.vec_c &&

@@ -329,3 +329,43 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
     assert seen == 88          # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 4 transposes with the old-C variant
+
+
+def _unpadded_wide_stores(body):
+    """Buffer stores of more than 8 bytes whose data registers the very next instruction writes.  The compiler pads such
+    a pair with wait states only when the store has no scalar offset register; with one it takes the hazard not to
+    exist, and on this chip lanes then stored the next value (seen with an accumulator read-back right behind the
+    store).  The epilogues therefore keep the scalar offset at literal zero."""
+    bad = []
+    for i, t in enumerate(body):
+        m = re.match(r"buffer_store_dwordx[34] (v\[\d+:\d+\]), \S+ s\[\d+:\d+\], (\S+)", t)
+        if not m:
+            continue
+        j = i + 1
+        while j < len(body) and body[j].endswith(":"):
+            j += 1
+        if j < len(body) and body[j].startswith("v_") and not body[j].startswith("v_cmp"):
+            dst = body[j].split(None, 1)[1].split(",")[0]
+            if _vregs(dst) & _vregs(m.group(1)):
+                bad.append((t, body[j]))
+    return bad
+
+
+def test_wide_store_checker_sees_a_planted_pair():
+    body = ["buffer_store_dwordx4 v[16:19], v68, s[40:43], s0 offen nt", "v_accvgpr_read_b32 v16, a[4]", "s_endpgm"]
+    assert len(_unpadded_wide_stores(body)) == 1
+    body = ["buffer_store_dwordx4 v[16:19], v68, s[40:43], 0 offen sc1", "s_nop 1", "v_accvgpr_read_b32 v16, a[4]", "s_endpgm"]
+    assert not _unpadded_wide_stores(body)
+
+
+def test_no_wide_buffer_store_is_followed_by_a_write_to_its_data(asm_files):
+    seen = 0
+    for path in asm_files:
+        for name, body in _kernels(path).items():
+            stores = [t for t in body if t.startswith("buffer_store_dwordx")]
+            for t in stores:
+                # (no scalar offset register on any of them: that is what makes the compiler pad the pair)
+                assert re.search(r"s\[\d+:\d+\], 0 offen", t), (name, t)
+            assert not _unpadded_wide_stores(body), (name, _unpadded_wide_stores(body)[:2])
+            seen += bool(stores)
+    assert seen >= 64           # every x16 kernel stores C through a buffer
