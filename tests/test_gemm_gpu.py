@@ -460,6 +460,35 @@ def test_identity_and_ones_closed_forms_full_size(dtype, size):
     assert torch.all(C == 0.25 * n)
 
 
+def test_x16_c_whose_tile_span_passes_32_bit_offsets():
+    """The whole-tile epilogue of the x16 kernels addresses C through a buffer descriptor with 32-bit offsets.  With
+    ldc so large that one tile's span of C (256 columns x ldc x 2 bytes) passes 2 GiB the library must take the
+    element-wise epilogue instead: same values, and nothing written outside the m x n window."""
+    import torch
+    import gemm_mmbo_amd as G
+    m, n, k = 256, 256, 64
+    ldc = (1 << 22) + 64                                  # 256 * ldc * 2 bytes > 2^31
+    cid = _x16_ids(F16)[0]
+    assert G.config_info(F16, cid)["macro_tile_n"] == 256
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77)
+    A = (torch.randn(m * k, device="cuda", generator=gen) * 0.1).half()
+    B = (torch.randn(k * n, device="cuda", generator=gen) * 0.1).half()
+    C = torch.zeros(ldc * n, device="cuda", dtype=torch.float16)
+    Cv = C.view(n, ldc)
+    C0 = (torch.rand(n, m, device="cuda", generator=gen) * 2 - 1).half()
+    Cv[:, :m] = C0
+    Cv[:, m:m + 16] = 7.0                                 # sentinels right below the window
+    G.gemm(F16, 0, 0, m, n, k, 1.5, A, m, B, k, 0.5, C, ldc, cid)
+    torch.cuda.synchronize()
+    want = 1.5 * (B.view(n, k).float() @ A.view(k, m).float()) + 0.5 * C0.float()      # column-major C = row-major C^T
+    got = Cv[:, :m].float()
+    assert float((got - want).abs().max()) <= 2e-2 * float(want.abs().max())
+    assert bool((Cv[:, m:m + 16] == 7.0).all()) and float(Cv[:, m + 16:].abs().max()) == 0.0
+    del C, Cv
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
 def test_old_c_closed_form_where_c_leaves_with_the_streaming_hint(dtype):
     """8192 x 8192 x 4096 on the 256 x 256 tile is 1,024 tiles with k >= 4096: the shape class whose C is stored with the
