@@ -56,9 +56,10 @@ struct DgemmCfg {
 // C = alpha*acc + beta*C for one wavefront's FM x FN blocks; acc[i][j][e] is
 // C(wrow0 + 16*i + 8*(e/2) + 2*(lane/16) + e%2, wcol0 + 16*j + lane%16).  beta == 0 never reads C
 // (src/gemm/ref/Kernels.cpp:87); alpha*acc first, then fma(beta, C, .), as the reference's epilogue.
+// `early`: the old C of the whole wave tile, requested by the caller under the last stage's MFMAs (dgemm_old_c), or null.
 template <int FM, int FN>
 __device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmArgs &args, uint32_t wrow0,
-                                        uint32_t wcol0, uint32_t batch, int lane)
+                                        uint32_t wcol0, uint32_t batch, int lane, const f64x2 (*early)[2] = nullptr)
 {
     const uint32_t m = args.m, n = args.n, ldc = args.ldc;
     const double alpha = args.alpha_d, beta = args.beta_d;
@@ -78,6 +79,11 @@ __device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmAr
                 f64x2 c[HB][2];
 #pragma unroll
                 for (int b = 0; b < HB; ++b) {
+                    if (early) {
+                        c[b][0] = early[b0 + b][0];
+                        c[b][1] = early[b0 + b][1];
+                        continue;
+                    }
                     const double *p = p0 + (size_t)((b0 + b) / FM) * 16 * ldc + ((b0 + b) % FM) * 16;
                     c[b][0] = *reinterpret_cast<const f64x2 *>(p);
                     c[b][1] = *reinterpret_cast<const f64x2 *>(p + 8);
@@ -134,7 +140,10 @@ __device__ inline void dgemm_write_back(const f64x4 (&acc)[FM][FN], const GemmAr
         }
 }
 
-template <bool TA, bool TB, int BM, int BN, int BK, int WM, int WN>
+// OLD_C_EARLY: the variant for beta != 0 that requests the wave tile's old C under the last stage's MFMAs (wave tiles of at
+// most four blocks).  A kernel of its own, picked by the host: the 32 registers per lane it holds the old C in take the
+// work-groups per CU from five to four, which calls without C to read would pay for nothing (1024^3, beta = 0: -1 %).
+template <bool TA, bool TB, int BM, int BN, int BK, int WM, int WN, bool OLD_C_EARLY = false>
 // Eight wavefronts with wave tiles of at most eight blocks (64 accumulator registers, two loader chunks per
 // operand) are held to 128 registers per lane so that two work-groups share a CU (the second argument is
 // wavefronts per SIMD); the others get 256.
@@ -242,9 +251,30 @@ dgemm_kernel(const GemmArgs args)
             cur ^= 1;
         }
     }
+    // Old C under the last stage's MFMAs (OLD_C_EARLY): requested at the top of the last stage -- no load follows it, so
+    // nothing in the loop waits for it -- and the epilogue finds it in registers instead of starting with one memory
+    // latency.  With five (now four) work-groups sharing a CU that latency was supposed to hide under the others' MFMAs;
+    // measured on the reference's HPL shape (44160 x 2048 x 384 NT, alpha = -1, beta = 1) it did not: 1,150 -> 1,088 us.
+    constexpr bool EARLY_C = OLD_C_EARLY && FM * FN <= 4;
+    [[maybe_unused]] f64x2 old_c[EARLY_C ? FM * FN : 1][2];
+    [[maybe_unused]] bool have_old_c = false;
     for (; it < n_iter; ++it) {
         const bool more = it + 1 < n_iter;
         if (more) load_stage(it + 1);
+        if constexpr (EARLY_C) {
+            const uint32_t wrow0 = row0 + wm * Cfg::TM, wcol0 = col0 + wn * Cfg::TN;
+            if (!more && args.beta_d != 0.0 && args.vec_c && wrow0 + FM * 16 <= args.m && wcol0 + FN * 16 <= args.n) {
+                const double *p0 = static_cast<const double *>(args.C) + (int64_t)batch * args.strideC +
+                                   (size_t)(wcol0 + (lane & 15)) * args.ldc + wrow0 + 2 * (lane >> 4);
+#pragma unroll
+                for (int b = 0; b < FM * FN; ++b) {
+                    const double *p = p0 + (size_t)(b / FM) * 16 * args.ldc + (b % FM) * 16;
+                    old_c[b][0] = *reinterpret_cast<const f64x2 *>(p);
+                    old_c[b][1] = *reinterpret_cast<const f64x2 *>(p + 8);
+                }
+                have_old_c = true;
+            }
+        }
 
         multiply_stage(lds + cur * Cfg::STAGE_BYTES);
 
@@ -257,6 +287,12 @@ dgemm_kernel(const GemmArgs args)
         cur ^= 1;
     }
 
+    if constexpr (EARLY_C) {
+        if (have_old_c) {
+            dgemm_write_back<FM, FN>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, lane, old_c);
+            return;
+        }
+    }
     dgemm_write_back<FM, FN>(acc, args, row0 + wm * Cfg::TM, col0 + wn * Cfg::TN, batch, lane);
 }
 

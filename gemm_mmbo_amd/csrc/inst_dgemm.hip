@@ -14,11 +14,15 @@ namespace mmbo {
 namespace {
 constexpr TileRow R = kTilesF64[MMBO_TILE];
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool OLD_C_EARLY = false>
 hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
     using Cfg = DgemmCfg<TA, TB, R.bm, R.bn, R.bk, R.wm, R.wn>;
-    auto kernel = dgemm_kernel<TA, TB, R.bm, R.bn, R.bk, R.wm, R.wn>;
+    // beta != 0 on a tile whose wave tiles have at most four blocks: the variant that requests the old C under the last stage
+    if constexpr (!OLD_C_EARLY && Cfg::FM * Cfg::FN <= 4) {
+        if (args.beta_d != 0.0 && args.vec_c) return launch_one<TA, TB, true>(args, stream);
+    }
+    auto kernel = dgemm_kernel<TA, TB, R.bm, R.bn, R.bk, R.wm, R.wn, OLD_C_EARLY>;
     static std::atomic<bool> attr_set[64];           // zero-initialised; several host threads may race to set it: harmless
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
