@@ -47,6 +47,7 @@ struct GemmArgs {
     uint32_t batch_xcd;     // 1: every problem of the batch runs on one XCD (batch_xcd_remap)
     uint32_t c_prefetch;    // 1: beta != 0 and the old C may be fetched into freed LDS ring buffers ahead of the epilogue
     uint32_t c_stream;      // 1: C leaves with the non-temporal hint (x16 kernel; long k, many rounds of tiles)
+    uint32_t line_rows;     // 1: A, B, their leading dimensions and batch strides are multiples of a 128-byte memory line
 };
 
 // Linear work-group id -> (tile row, tile column).

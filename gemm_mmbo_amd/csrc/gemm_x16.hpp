@@ -330,8 +330,10 @@ struct X16Cfg {
 // OLD_C_AHEAD: the variant for beta != 0 that fetches a tile's old C into LDS under the tile's last four slices (see c_ahead
 // below; both load schedules).  A kernel of its own, chosen by the host: with the code in the one kernel, calls that have no C to read paid
 // 1.5-3 % on short-k and mid-size shapes for tails that had grown.
+// BOTH_EVEN: the variant for two k-contiguous operands (TN) whose rows start on memory lines: both operands' pairs on the
+// even iterations (see BOTH below).  A kernel of its own, chosen by the host.
 template <typename T, bool TA, bool TB, int BM, int BN, int WM, int WN, int DEPTH, bool PAIR = (TA || !TB),
-          int EVEN_OP = (TA ? 0 : 1), bool OLD_C_AHEAD = false>
+          int EVEN_OP = (TA ? 0 : 1), bool OLD_C_AHEAD = false, bool BOTH_EVEN = false>
 __global__ void __launch_bounds__(WM * WN * 64)
 gemm_x16_kernel(const GemmArgs args)
 {
@@ -344,6 +346,14 @@ gemm_x16_kernel(const GemmArgs args)
     using FragB = typename Cfg::FragB;
     constexpr int FM = Cfg::FM, FN = Cfg::FN, BK = Cfg::BK, BATCH = Cfg::BATCH, NACC = Cfg::NACC, ESZ = Cfg::ESZ;
     [[maybe_unused]] constexpr int MPF = Cfg::MPF;
+    // Both operands k-contiguous (TN) on a ring of five buffers: the even iterations fetch the pair of slices s+4, s+5 of BOTH
+    // operands and the odd ones nothing.  Alternating the operands, the odd iterations' pairs (s+4, s+5 with s odd) start on an
+    // odd slice and so straddle two memory lines: half-line requests for half of the traffic.  The waits are the same either
+    // way -- the loads of the last two iterations may stay in flight -- and so is the shortest lead (a pair's first slice is
+    // requested two to three slices before it is needed).  Measured (fp16, us): 64 x 512^3 27.1 -> 25.0, 2048^3 21.9 -> 20.7,
+    // 4096^3 105.8 -> 101.5, 8192^3 777 -> 765.  Only where every row of A and B starts on a memory line (BOTH_EVEN, the host's
+    // choice): with rows that straddle lines anyway the bunched requests cost 7 % (8192 x 8192 x 8200, lda = ldb = 8200).
+    constexpr bool BOTH = BOTH_EVEN && PAIR && TA && !TB && DEPTH == 5;
 
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -481,15 +491,22 @@ gemm_x16_kernel(const GemmArgs args)
         constexpr int load_mode = decltype(LOAD)::value;          // 0 none, 1 always, 2 if `load` (and `load2`)
         constexpr int par = decltype(PAR)::value;
         constexpr int opn = par ^ EVEN_OP;                         // paired mode: the operand this iteration fetches
-        constexpr int LOP = opn == 0 ? TileA::LPW : TileB::LPW;   // and its loads per slice
+        constexpr int LX = EVEN_OP == 0 ? TileA::LPW : TileB::LPW, LY = EVEN_OP == 0 ? TileB::LPW : TileA::LPW;
+        // and its loads per slice (BOTH: the even operand's loads, then the other one's; the odd iterations fetch nothing)
+        constexpr int LOP = BOTH ? (par == 0 ? LX + LY : 0) : (opn == 0 ? TileA::LPW : TileB::LPW);
+        constexpr int load_mode_here = (BOTH && par == 1) ? 0 : load_mode;
         const int pbuf = lbuf == 0 ? DEPTH - 1 : lbuf - 1;        // buffer of slice s+DEPTH-1
         const uint32_t t = lds_base + nbuf * Cfg::SLICE_BYTES;
         // LDS destinations of this iteration's loads, worked out here, once (the empty asm pins them to scalar registers
         // at this point: otherwise the compiler recomputes them next to every load, between two MFMAs)
         uint32_t dst_x0 = op_dst(std::integral_constant<int, opn>{}, pbuf), dst_x1 = op_dst(std::integral_constant<int, opn>{}, lbuf);
         uint32_t dst_a = op_dst(std::integral_constant<int, 0>{}, lbuf), dst_b = op_dst(std::integral_constant<int, 1>{}, lbuf);
-        if constexpr (load_mode != 0 && PAIR) asm volatile("" : "+s"(dst_x0), "+s"(dst_x1));
-        if constexpr (load_mode != 0 && !PAIR) asm volatile("" : "+s"(dst_a), "+s"(dst_b));
+        // (BOTH: the other operand's two destinations)
+        [[maybe_unused]] uint32_t dst_y0 = op_dst(std::integral_constant<int, 1 - EVEN_OP>{}, pbuf),
+                                  dst_y1 = op_dst(std::integral_constant<int, 1 - EVEN_OP>{}, lbuf);
+        if constexpr (load_mode_here != 0 && PAIR) asm volatile("" : "+s"(dst_x0), "+s"(dst_x1));
+        if constexpr (load_mode_here != 0 && BOTH) asm volatile("" : "+s"(dst_y0), "+s"(dst_y1));
+        if constexpr (load_mode_here != 0 && !PAIR) asm volatile("" : "+s"(dst_a), "+s"(dst_b));
         // old C ahead of the epilogue: this iteration's groups c_first .. c_first + C_PER_SLICE - 1 go to buffer lbuf (the
         // one this slice left; no operand load goes there any more), one after every eighth MFMA
         [[maybe_unused]] const uint32_t c_dst = lds_base + (uint32_t)lbuf * Cfg::SLICE_BYTES + wave * (Cfg::C_PER_SLICE * 1024);
@@ -506,14 +523,16 @@ gemm_x16_kernel(const GemmArgs args)
             // lines, one MFMA later.  Unpaired: load l after MFMA number (2l+1) * NMFMA / (2 * BATCH): evenly spaced, none
             // first or last.  Where exactly one load follows the MFMA, its LDS destination goes into M0 BEFORE the MFMA and the
             // load itself after it: the MFMA is the wait state a write to M0 needs, and the load costs two instructions.
-            constexpr int LIM = PAIR ? LOP : BATCH;
+            constexpr int LIM = PAIR ? (LOP > 0 ? LOP : 1) : BATCH;
             constexpr int l0 = loads_before_slot(LIM, NMFMA, m), l1 = loads_before_slot(LIM, NMFMA, m + 1),
                           p0 = m == 0 ? 0 : loads_before_slot(LIM, NMFMA, m - 1);
-            constexpr int n_first = load_mode != 0 ? l1 - l0 : 0, n_second = (load_mode != 0 && PAIR) ? l0 - p0 : 0;
+            constexpr int n_first = load_mode_here != 0 ? l1 - l0 : 0, n_second = (load_mode_here != 0 && PAIR) ? l0 - p0 : 0;
             static_assert(!PAIR || m + 1 < NMFMA || n_first == 0, "the last MFMA slot cannot start a pair of loads");
             constexpr bool single = n_first + n_second == 1;
             if constexpr (single) {
-                if constexpr (n_second == 1) set_lds_destination(dst_x1 + p0 * 1024);
+                if constexpr (BOTH && n_second == 1) set_lds_destination(p0 < LX ? dst_x1 + p0 * 1024 : dst_y1 + (p0 - LX) * 1024);
+                else if constexpr (BOTH) set_lds_destination(l0 < LX ? dst_x0 + l0 * 1024 : dst_y0 + (l0 - LX) * 1024);
+                else if constexpr (n_second == 1) set_lds_destination(dst_x1 + p0 * 1024);
                 else if constexpr (PAIR) set_lds_destination(dst_x0 + l0 * 1024);
                 else if constexpr (l0 < TileA::LPW) set_lds_destination(dst_a + l0 * 1024);
                 else set_lds_destination(dst_b + (l0 - TileA::LPW) * 1024);
@@ -544,11 +563,17 @@ gemm_x16_kernel(const GemmArgs args)
             constexpr std::bool_constant<single> DESTINATION_SET{};
             static_for<n_second>([&](auto LL) {
                 constexpr int l = p0 + decltype(LL)::value;
-                if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::true_type{}, dst_x1, DESTINATION_SET);
+                if constexpr (BOTH && l >= LX) {
+                    if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, 1 - EVEN_OP>{}, std::integral_constant<int, l - LX>{}, std::true_type{}, dst_y1, DESTINATION_SET);
+                } else {
+                    if (load_mode == 1 || load2) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::true_type{}, dst_x1, DESTINATION_SET);
+                }
             });
             static_for<n_first>([&](auto LL) {
                 constexpr int l = l0 + decltype(LL)::value;
-                if constexpr (PAIR) {
+                if constexpr (BOTH && l >= LX) {
+                    if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, 1 - EVEN_OP>{}, std::integral_constant<int, l - LX>{}, std::false_type{}, dst_y0, DESTINATION_SET);
+                } else if constexpr (PAIR) {
                     if (load_mode == 1 || load) issue_op_load(std::integral_constant<int, opn>{}, std::integral_constant<int, l>{}, std::false_type{}, dst_x0, DESTINATION_SET);
                 } else {
                     if (load_mode == 1 || load) issue_load(std::integral_constant<int, l>{}, dst_a, dst_b, DESTINATION_SET);
@@ -569,7 +594,8 @@ gemm_x16_kernel(const GemmArgs args)
         // the cursors move past what this iteration requested (past the end of k in the last iterations: never used again).
         // The paired tail moves them itself, behind its choice between two copies of the slice: a cursor that is changed on
         // one side of a branch only comes out of the merge in vector registers, where a buffer load cannot take it.
-        if constexpr (load_mode == 1 && PAIR) advance_op(std::integral_constant<int, opn>{}, 2);
+        if constexpr (load_mode_here == 1 && PAIR) advance_op(std::integral_constant<int, opn>{}, 2);
+        if constexpr (load_mode_here == 1 && BOTH) advance_op(std::integral_constant<int, 1 - EVEN_OP>{}, 2);
         if constexpr (load_mode != 0 && !PAIR) {
             advance(curA, (uint64_t)stepA);
             advance(curB, (uint64_t)stepB);
@@ -681,13 +707,19 @@ gemm_x16_kernel(const GemmArgs args)
         constexpr int X_PAIRED = DEPTH == 5 ? 4 : 2;                     // X's slices below this go out in pairs
         pro_pair(OPX, NLA, 0);
         pro_pair(OPY, NLB, 0);
-        if constexpr (X_PAIRED == 4) pro_pair(OPX, NLA, 2);
+        if constexpr (BOTH) {
+            // (both operands on the even iterations: slices 0 .. 3 of both here, all in pairs; iteration 0 brings 4 and 5)
+            pro_pair(OPX, NLA, 2);
+            pro_pair(OPY, NLB, 2);
+        } else {
+            if constexpr (X_PAIRED == 4) pro_pair(OPX, NLA, 2);
 #pragma unroll
-        for (int q = 2; q < DEPTH; ++q) {
-            if (q >= X_PAIRED && q < DEPTH - 1) pro_one(OPX, NLA, q);
-            pro_one(OPY, NLB, q);
+            for (int q = 2; q < DEPTH; ++q) {
+                if (q >= X_PAIRED && q < DEPTH - 1) pro_one(OPX, NLA, q);
+                pro_one(OPY, NLB, q);
+            }
         }
-        constexpr int PRO = (DEPTH - 1) * LA + DEPTH * LB;               // loads per thread in the prologue
+        constexpr int PRO = BOTH ? (DEPTH - 1) * (LA + LB) : (DEPTH - 1) * LA + DEPTH * LB;       // loads per thread in the prologue
         acc_zero<NACC>();                                                // (while the first slices are on their way)
         if (n_slice >= DEPTH) MMBO_WAIT_VM(PRO - 2 * BATCH); else MMBO_WAIT_VM(0);
         MMBO_BARRIER();                                                  // slices 0 and 1 resident
@@ -699,7 +731,8 @@ gemm_x16_kernel(const GemmArgs args)
         auto steady_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             constexpr int par = decltype(PAR)::value;
             constexpr int own = 2 * (par == 0 ? LA : LB), other = 2 * (par == 0 ? LB : LA);
-            constexpr int KEEP = own * ((DEPTH - 3 + 1) / 2) + other * ((DEPTH - 3) / 2);
+            // (BOTH, five buffers: this iteration and the one before it, of which one fetched both operands' pairs and one nothing)
+            constexpr int KEEP = BOTH ? 2 * (LA + LB) : own * ((DEPTH - 3 + 1) / 2) + other * ((DEPTH - 3) / 2);
             static_assert(KEEP < 64, "more loads in flight than vmcnt can count");
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
             mfma_and_read(std::integral_constant<int, 1>{}, PAR, ca, cb, na, nb, nbuf, true, true, buf, std::false_type{}, 0);
@@ -712,10 +745,10 @@ gemm_x16_kernel(const GemmArgs args)
         int hist[2] = {0, 0};
         auto tail_step = [&](auto PAR, int s, FragA &ca, FragB &cb, FragA &na, FragB &nb) {
             constexpr int par = decltype(PAR)::value;
-            constexpr int LOP = par == 0 ? LA : LB;
+            constexpr int LOP = BOTH ? (par == 0 ? LA + LB : 0) : (par == 0 ? LA : LB);
             constexpr int G = gcd_of(LA, LB);                            // every count below is a multiple of it
             const int nbuf = buf + 1 == DEPTH ? 0 : buf + 1;
-            const bool load = s + DEPTH - 1 < n_slice, load2 = s + DEPTH < n_slice;
+            const bool load = LOP != 0 && s + DEPTH - 1 < n_slice, load2 = LOP != 0 && s + DEPTH < n_slice;
             // the last four slices carry the old C of the epilogue (no operand load is left to issue by then)
             // (a copy of the slice of its own, chosen once per slice: a test in front of each of its loads cost the tails of
             // short-k problems without C to fetch 1-3 %)
@@ -729,12 +762,16 @@ gemm_x16_kernel(const GemmArgs args)
             } else {
                 mfma_and_read(std::integral_constant<int, 2>{}, PAR, ca, cb, na, nb, nbuf, load, load2, buf, std::false_type{}, 0);
             }
-            advance_op(std::integral_constant<int, par ^ EVEN_OP>{}, 2);
+            if constexpr (BOTH) {
+                if constexpr (par == 0) { advance_op(OPX, 2); advance_op(OPY, 2); }
+            } else {
+                advance_op(std::integral_constant<int, par ^ EVEN_OP>{}, 2);
+            }
             MMBO_WAIT_LGKM0();
             const int cur = ((load ? 1 : 0) + (load2 ? 1 : 0)) * LOP +
                             (c_first >= 0 ? max(0, min(Cfg::C_PER_SLICE, Cfg::C_GROUPS - c_first)) : 0);
             const int keep = cur + hist[0] + (DEPTH >= 6 ? hist[1] : 0);
-            constexpr int KMAX0 = 2 * (LA > LB ? LA : LB) * 3, KC3 = OLD_C_AHEAD ? 3 * Cfg::C_PER_SLICE : 0;
+            constexpr int KMAX0 = BOTH ? 2 * (LA + LB) : 2 * (LA > LB ? LA : LB) * 3, KC3 = OLD_C_AHEAD ? 3 * Cfg::C_PER_SLICE : 0;
             constexpr int KMAX = ((KMAX0 > KC3 ? KMAX0 : KC3) + G - 1) / G * G;
             bool waited = false;
             static_for<KMAX / G>([&](auto Q) {
@@ -752,8 +789,8 @@ gemm_x16_kernel(const GemmArgs args)
         for (; s + 1 + DEPTH < n_slice; s += 2) {
             steady_step(EVEN, s, fa[0], fb[0], fa[1], fb[1]);
             steady_step(ODD, s + 1, fa[1], fb[1], fa[0], fb[0]);
-            hist[0] = 2 * LB;
-            hist[1] = 2 * LA;
+            hist[0] = BOTH ? 0 : 2 * LB;
+            hist[1] = BOTH ? 2 * (LA + LB) : 2 * LA;
         }
         for (; s < n_slice; s += 2) {
             tail_step(EVEN, s, fa[0], fb[0], fa[1], fb[1]);

@@ -16,15 +16,20 @@ namespace {
 using ElemT = typename std::conditional<MMBO_DTYPE == 0, float, half_t>::type;
 constexpr RingRow R = kX16Tiles[MMBO_TILE];
 
-template <bool TA, bool TB, int WM, int WN, bool OLD_C = false>
+template <bool TA, bool TB, int WM, int WN, bool OLD_C = false, bool BOTH_EVEN = false>
 hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
 {
     using Cfg = X16Cfg<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth>;
     // beta != 0 on fp16 (args.c_prefetch): the variant that fetches the old C ahead of the epilogue, where the tile has one
     if constexpr (!OLD_C && Cfg::C_PREFETCH) {
-        if (args.c_prefetch) return launch_one<TA, TB, WM, WN, true>(args, stream);
+        if (args.c_prefetch) return launch_one<TA, TB, WM, WN, true, BOTH_EVEN>(args, stream);
     }
-    auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth, (TA || !TB), (TA ? 0 : 1), OLD_C>;
+    // TN on a ring of five buffers with every row of A and B on a memory line (args.line_rows): both operands' pairs of
+    // slices on the even iterations
+    if constexpr (!BOTH_EVEN && TA && !TB && R.depth == 5) {
+        if (args.line_rows) return launch_one<TA, TB, WM, WN, OLD_C, true>(args, stream);
+    }
+    auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth, (TA || !TB), (TA ? 0 : 1), OLD_C, BOTH_EVEN>;
     static std::atomic<bool> attr_set[64];           // zero-initialised; several host threads may race to set it: harmless
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);

@@ -275,6 +275,36 @@ def test_x16_kernel_old_c_fetched_under_the_last_slices(ta, tb):
     assert ran == 48
 
 
+@pytest.mark.parametrize("dtype", [F32, F16], ids=NAMES.get)
+def test_x16_tn_with_both_operands_fetched_on_the_even_slices(dtype):
+    """TN on a ring of five buffers, every row of A and B starting on a 128-byte memory line (k a multiple of 64 fp16 / 32
+    fp32 elements, tight leading dimensions): the kernel variant that fetches both operands' pairs of slices on the even
+    iterations.  Even slice counts from below the ring depth to several steady iterations, with and without the old C
+    under the last slices (beta), several tiles per resident work-group, batches; and the same shapes with lda or ldb off
+    the line, which must take the alternating variant and give the same values."""
+    import gemm_mmbo_amd as G
+    ids = [c for c in _x16_ids(dtype) if G.config_info(dtype, c)["split_k"] == 1]
+    bk = 16 if dtype == F32 else 32
+    line = 128 // (4 if dtype == F32 else 2)                  # elements per memory line
+    ran = 0
+    for cid in ids:
+        d = G.config_info(dtype, cid)
+        bm, bn = d["macro_tile_m"], d["macro_tile_n"]
+        if d["lds_bytes"] // ((bm + bn) * 64) != 5:
+            continue
+        for slices, (tm, tn, batch), beta in ((2, (1, 1, 1), 0.0), (4, (1, 1, 2), 0.5), (6, (1, 2, 1), 0.0), (8, (2, 1, 1), 0.5),
+                                              (10, (1, 1, 1), 0.5), (14, (3, 2, 1), 0.0), (16, (1, 1, 2), 0.5), (36, (1, 1, 1), 0.5)):
+            m, n, k = bm * tm, bn * tn, bk * slices
+            assert k % line == 0
+            for pad in (0, 8):
+                p = U.Problem(dtype, 1, 0, m, n, k, 1.25, beta, lda=k + pad, ldb=k + (0 if slices % 4 else pad), batch=batch,
+                              seed=900 + cid + slices, dist="normal" if dtype == F16 else "uniform",
+                              c_fill="uniform" if beta else "nan")
+                _run_and_check(p, cid, label=f"{d['name']} TN {m}x{n}x{k} b{batch} lda {k + pad}")
+                ran += 1
+    assert ran == 5 * 8 * 2
+
+
 def test_x16_kernel_chip_block_order_and_refusals():
     """Grids of at least 16 x 16 tiles of 256 x 256 walk the tiles in chip-wide blocks: whole blocks, blocks plus a
     ragged border of tiles, against the oracle.  Unaligned operands are taken, a contiguous dimension shorter than one

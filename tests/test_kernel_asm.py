@@ -328,7 +328,9 @@ def test_x16_kernels_claim_exactly_their_accumulation_registers(asm_files):
             assert used == set(range(len(used))) and len(used) in (64, 128, 256), (name, len(used))
             assert agprs == len(used), (name, agprs, len(used))
             seen += 1
-    assert seen == 88          # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 4 transposes with the old-C variant
+    # 8 tiles x 2 element types x 4 transposes, + 6 fp16 tiles x 4 transposes with the old-C variant, + the TN variant with both
+    # operands on the even slices for the 5 tiles with five ring buffers x 2 element types, + its 5 fp16 old-C forms
+    assert seen == 88 + 10 + 5
 
 
 def _unpadded_wide_stores(body):
