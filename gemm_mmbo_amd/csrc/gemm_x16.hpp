@@ -327,6 +327,10 @@ struct X16Cfg {
 // EVEN_OP: the operand (0 = A, 1 = B) that paired mode fetches on even iterations.  Measured at 8192^3, against
 // unpaired: NN and TT +1.0 to +1.5 % with the k-contiguous operand on the even iterations and -1.5 % with the other
 // one, TN (both k-contiguous) +0.8 % with four wavefronts and +2.5 % with eight, NT (neither) -1.3 %.
+// What decides it is where a pair starts: iteration s fetches slices s+DEPTH-1 and s+DEPTH, two halves of the same 128-byte
+// lines only when the first of them is even -- s even for a ring of five buffers, s odd for a ring of six.  The launcher
+// therefore gives the k-contiguous operand the even iterations on five buffers and the odd ones on six (six buffers, fp16:
+// 3072^3 NN on the 192 x 192 tile 52.2 -> 50.3 us, 1024 x 1024 x 4096 on 64 x 64 21.1 -> 18.9, 2048 x 1024 x 4096 on 128 x 64 27.2 -> 25.3).
 // OLD_C_AHEAD: the variant for beta != 0 that fetches a tile's old C into LDS under the tile's last four slices (see c_ahead
 // below; both load schedules).  A kernel of its own, chosen by the host: with the code in the one kernel, calls that have no C to read paid
 // 1.5-3 % on short-k and mid-size shapes for tails that had grown.

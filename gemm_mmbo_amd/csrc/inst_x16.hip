@@ -29,7 +29,10 @@ hipError_t launch_one(const GemmArgs &args, hipStream_t stream)
     if constexpr (!BOTH_EVEN && TA && !TB && R.depth == 5) {
         if (args.line_rows) return launch_one<TA, TB, WM, WN, OLD_C, true>(args, stream);
     }
-    auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth, (TA || !TB), (TA ? 0 : 1), OLD_C, BOTH_EVEN>;
+    // the k-contiguous operand goes to the iterations whose pair of slices starts on an even slice (whole memory lines): the
+    // even ones on a ring of five buffers, the odd ones on a ring of six
+    constexpr int EVEN_OP = R.depth == 6 ? (TA ? 1 : 0) : (TA ? 0 : 1);
+    auto kernel = gemm_x16_kernel<ElemT, TA, TB, R.bm, R.bn, WM, WN, R.depth, (TA || !TB), EVEN_OP, OLD_C, BOTH_EVEN>;
     static std::atomic<bool> attr_set[64];           // zero-initialised; several host threads may race to set it: harmless
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
