@@ -302,7 +302,18 @@ def test_x16_tn_with_both_operands_fetched_on_the_even_slices(dtype):
                               c_fill="uniform" if beta else "nan")
                 _run_and_check(p, cid, label=f"{d['name']} TN {m}x{n}x{k} b{batch} lda {k + pad}")
                 ran += 1
-    assert ran == 5 * 8 * 2
+        # odd slice counts, a partial last slice and edge tiles under the same variant: the leading dimensions padded up to
+        # a whole number of memory lines
+        for (m, n, slices, kt, beta, batch) in ((bm, bn, 5, 0, 0.5, 1), (bm + 8, 2 * bn - 8, 7, 0, 0.0, 1), (bm, bn, 9, 5, 0.5, 2),
+                                                (2 * bm - 8, bn + 8, 13, bk - 1, 0.0, 1), (bm, bn, 1, 0, 0.5, 1), (bm, bn, 3, 3, 0.0, 1)):
+            k = bk * slices + kt
+            ld = -(-k // line) * line
+            p = U.Problem(dtype, 1, 0, m, n, k, -0.75, beta, lda=ld, ldb=ld, ldc=m + 8, batch=batch, seed=950 + cid + slices,
+                          dist="normal" if dtype == F16 else "uniform", c_fill="uniform" if beta else "nan")
+            assert (p.sa * (4 if dtype == F32 else 2)) % 128 == 0
+            _run_and_check(p, cid, label=f"{d['name']} TN {m}x{n}x{k} b{batch} ld {ld}")
+            ran += 1
+    assert ran == 5 * (8 * 2 + 6)
 
 
 def test_x16_kernel_chip_block_order_and_refusals():
