@@ -198,8 +198,11 @@ def skinny_legs(G, torch, steps, warmup):
             us = timed_launches(torch, stream, lambda: G.gemm(dtype, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m, cid, stream),
                                 max(steps, 200), max(warmup, 20), groups=10, settle_min_ms=30.0, settle_max_ms=200.0)["median_ms"] * 1e3
             nbytes = (m * k + k * n + m * n) * esz
+            # a plain streaming kernel with the same bytes read and written, on this box, launched the same way
+            stream_us = G.probe_stream((m * k + k * n) * esz, m * n * esz, 50) * 1e6
             out[f"{dname}_{m}x{n}x{k}"] = {"us": round(us, 2), "algorithmic_GBps": round(nbytes / us * 1e-3, 1),
                                             "frac_of_hbm_peak": round(nbytes / us * 1e-3 / 8000.0, 4),
+                                            "stream_kernel_same_bytes_us": round(stream_us, 2),
                                             "tflops": round(2.0 * m * n * k / us * 1e-6, 1),
                                             "tile_config": G.config_info(dtype, cid)["name"]}
     return out
@@ -265,6 +268,10 @@ def config_legs(G, torch, steps, warmup):
         out[key] = {"us": round(us, 1), "tflops": round(tf, 1),
                     "frac_of_peak": round(tf / PEAK_TFLOPS["f16" if dtype == G.F16 else "f32"], 4),
                     "algorithmic_GBps": round(gbps, 1), "tile_config": G.config_info(dtype, cid)["name"]}
+        if batch > 1:
+            # the memory-bound one: a plain streaming kernel with the same bytes read (A, B, old C) and written, on this box
+            out[key]["stream_kernel_same_bytes_us"] = round(
+                G.probe_stream(batch * (m * k + k * n + (m * n if beta != 0 else 0)) * esz, batch * m * n * esz, 50, in_place=beta != 0) * 1e6, 1)
         del A, B, C
     return out
 

@@ -21,7 +21,7 @@ EXPORTS = (
     "mmbo_gemm", "mmbo_gemm_strided_batched", "mmbo_gemm_strided_batched_static_workspace", "mmbo_static_workspace_bytes",
     "mmbo_num_configs", "mmbo_config_info", "mmbo_select_config",
     "mmbo_wg_remap", "mmbo_chip_block_remap", "mmbo_batch_xcd_remap", "mmbo_release_workspace", "mmbo_release_stream_workspace", "mmbo_workspace_info",
-    "mmbo_probe_mfma_ceiling", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
+    "mmbo_probe_mfma_ceiling", "mmbo_probe_stream", "mmbo_status_string", "mmbo_last_hip_error", "mmbo_version",
 )
 
 
@@ -82,6 +82,8 @@ def lib():
         dp = ctypes.POINTER(ctypes.c_double)
         L.mmbo_probe_mfma_ceiling.argtypes = [ci, ci, dp, dp]
         L.mmbo_probe_mfma_ceiling.restype = ci
+        L.mmbo_probe_stream.argtypes = [sz, sz, ci, ci, dp]
+        L.mmbo_probe_stream.restype = ci
         L.mmbo_status_string.argtypes = [ci]
         L.mmbo_status_string.restype = ctypes.c_char_p
         L.mmbo_last_hip_error.restype = ci
@@ -189,6 +191,14 @@ def chip_block_remap(linear_id, nwg0, nwg1):
     a, b = ctypes.c_uint(0), ctypes.c_uint(0)
     _check(lib().mmbo_chip_block_remap(linear_id, nwg0, nwg1, ctypes.byref(a), ctypes.byref(b)))
     return a.value, b.value
+
+
+def probe_stream(read_bytes, write_bytes, launches=20, in_place=False):
+    """Seconds per launch of a plain streaming kernel that reads and writes that many bytes on the current device (in_place:
+    the writes go over the first of the bytes read, as an update of C with beta != 0 does)."""
+    t = ctypes.c_double(0.0)
+    _check(lib().mmbo_probe_stream(int(read_bytes), int(write_bytes), 1 if in_place else 0, int(launches), ctypes.byref(t)))
+    return t.value
 
 
 def probe_mfma_ceiling(dtype, random_operands=True):

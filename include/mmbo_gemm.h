@@ -181,6 +181,17 @@ int mmbo_workspace_info(size_t *slots, size_t *bytes);
  * hundred KB; takes some tens of milliseconds. */
 int mmbo_probe_mfma_ceiling(int dtype, int random_operands, double *tflops, double *shader_mhz);
 
+/* Measures what a plain streaming kernel sustains on the current device with the byte counts of a memory-bound GEMM:
+ * read_bytes read from one buffer and write_bytes written per launch (multiples of 16; either may be 0) -- to a second
+ * buffer, or, with in_place set, over the first write_bytes of what was read, the way beta != 0 updates C --,
+ * whole-chip grid-stride loops, `launches` launches back to back, the fastest of five such groups.  Returns seconds
+ * per launch: the measured counterpart of the nominal 8 TB/s for shapes whose bound is memory (the batched and the
+ * skinny benchmark configs), as mmbo_probe_mfma_ceiling is of the nominal matrix peak.  Buffers of up to a few hundred
+ * MB stay in the last-level cache from launch to launch, as a GEMM's operands do in a benchmark loop.  The reference has
+ * no bandwidth figure at all (its harness reports GFLOP/s against a hard-coded peak, src/gemm/test.cc:87-88).
+ * Allocates and frees read_bytes + write_bytes. */
+int mmbo_probe_stream(size_t read_bytes, size_t write_bytes, int in_place, int launches, double *seconds_per_launch);
+
 const char *mmbo_status_string(int status);
 int mmbo_last_hip_error(void);       /* hipError_t of the last MMBO_ERR_HIP on this thread */
 const char *mmbo_version(void);

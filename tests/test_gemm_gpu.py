@@ -478,6 +478,24 @@ def test_batched_equals_looped_single_calls_bitwise():
     assert np.array_equal(dC.cpu().numpy().view(np.uint16), got.view(np.uint16))
 
 
+def test_stream_probe_reports_a_plausible_rate_and_refuses_bad_sizes():
+    """mmbo_probe_stream: a plain streaming kernel over given byte counts.  The rate it reports for a copy of 64 MiB
+    lies between what any HBM part of this class sustains and the nominal 8 TB/s plus what the last-level cache adds;
+    twice the bytes take longer; read-only and write-only runs work; sizes that are not whole 16-byte vectors are refused."""
+    import gemm_mmbo_amd as G
+    mib = 1 << 20
+    t1 = G.probe_stream(64 * mib, 64 * mib, 20)
+    t2 = G.probe_stream(256 * mib, 256 * mib, 10)
+    assert 1.0e12 < 128 * mib / t1 < 16.0e12, t1
+    assert t2 > 1.5 * t1
+    assert G.probe_stream(64 * mib, 0, 10) > 0 and G.probe_stream(0, 64 * mib, 10) > 0
+    assert G.probe_stream(96 * mib, 32 * mib, 10, in_place=True) > 0
+    for args in ((24, 16, 1), (16, 8, 1), (0, 0, 1), (16, 16, 0), (16, 32, 1, True)):
+        with pytest.raises(G.MmboError) as e:
+            G.probe_stream(*args)
+        assert e.value.status != 0
+
+
 # ------------------------------------------------------------------ size-independent properties at full size
 
 @pytest.mark.parametrize("dtype,size", [(F32, 4096), (F16, 8192)], ids=["f32-4096", "f16-8192"])
