@@ -52,6 +52,14 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise MmboError(-1, f"{LIB_PATH} is missing: run `python -m gemm_mmbo_amd.build` (needs hipcc); "
                                 "this package has no CPU or PyTorch fallback")
+        # PyTorch first, where there is one: its wheel brings a HIP runtime of its own under a different file name, and a process
+        # that has loaded the system's copy before (through this library) ends up with two runtimes, of which only the one
+        # loaded first finds a device for this library's calls -- on tensors the other one allocated.  Loaded after torch, the
+        # library binds to the runtime torch uses.
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         sz, ll, vp, ci, cu = ctypes.c_size_t, ctypes.c_longlong, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint
         L.mmbo_gemm.argtypes = [ci, ci, ci, sz, sz, sz, vp, vp, sz, vp, sz, vp, vp, sz, ci, vp]

@@ -247,19 +247,24 @@ extern "C" int mmbo_probe_stream(size_t read_bytes, size_t write_bytes, int in_p
         if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) break;
         const dim3 grid((unsigned)prop.multiProcessorCount * 4), block(256);
         const size_t r16 = read_bytes / 16, w16 = write_bytes / 16;
-        for (int i = 0; i < 10; ++i) hipLaunchKernelGGL(stream_probe_kernel<12>, grid, block, 0, nullptr, src, dst, r16, w16);
-        float best = 0.0f;
+        // (each launch's own status: the thread's last-error state may hold an error some earlier, unrelated call left behind)
+        const u32x4 *ksrc = src;
+        size_t kr = r16, kw = w16;
+        void *kargs[] = {&ksrc, &dst, &kr, &kw};
+        auto launch = [&]() { return hipLaunchKernel(reinterpret_cast<const void *>(stream_probe_kernel<12>), grid, block, kargs, 0, nullptr); };
         bool ok = true;
+        for (int i = 0; i < 10 && ok; ++i) ok = launch() == hipSuccess;
+        float best = 0.0f;
         for (int rep = 0; rep < 5 && ok; ++rep) {            // the fastest of five groups of `launches` back-to-back launches
             (void)hipEventRecord(e0, nullptr);
-            for (int i = 0; i < launches; ++i) hipLaunchKernelGGL(stream_probe_kernel<12>, grid, block, 0, nullptr, src, dst, r16, w16);
+            for (int i = 0; i < launches && ok; ++i) ok = launch() == hipSuccess;
             (void)hipEventRecord(e1, nullptr);
-            ok = hipEventSynchronize(e1) == hipSuccess;
+            ok = hipEventSynchronize(e1) == hipSuccess && ok;
             float ms = 0.0f;
             (void)hipEventElapsedTime(&ms, e0, e1);
             if (rep == 0 || ms < best) best = ms;
         }
-        if (!ok || best <= 0.0f || hipGetLastError() != hipSuccess) break;
+        if (!ok || best <= 0.0f) break;
         *seconds_per_launch = (double)best * 1e-3 / launches;
         rc = MMBO_OK;
     } while (false);

@@ -6,6 +6,8 @@ beta == 0 "never read C" rule, k = 0, strided batches, and size-independent prop
 ones, linearity in alpha/beta) at full size.  Tolerances are in tests/util.py:
 fp32 <= 1e-5*sqrt(K), fp16 <= 2e-2, relative to max(|exact|, rms(exact)).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -476,6 +478,27 @@ def test_batched_equals_looped_single_calls_bitwise():
                1.0, dC.data_ptr() + 2 * b * p.sc, p.ldc, cid)
     torch.cuda.synchronize()
     assert np.array_equal(dC.cpu().numpy().view(np.uint16), got.view(np.uint16))
+
+
+def test_package_imported_before_torch_still_reaches_the_device():
+    """A fresh process that touches the library before it imports torch: the Python layer must end up on the HIP runtime
+    torch uses (the wheel ships its own copy; with the system's copy loaded first the library's calls found no device)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "import gemm_mmbo_amd as G\n"
+            "assert G.num_configs(G.F16) > 0\n"
+            "import torch\n"
+            "m = n = k = 256\n"
+            "A = torch.ones(m * k, device='cuda', dtype=torch.float16); B = torch.ones(k * n, device='cuda', dtype=torch.float16)\n"
+            "C = torch.zeros(m * n, device='cuda', dtype=torch.float16)\n"
+            "G.gemm(G.F16, 0, 0, m, n, k, 1.0, A, m, B, k, 0.0, C, m)\n"
+            "torch.cuda.synchronize()\n"
+            "assert bool((C == k).all())\n"
+            "print('ok')\n") % root
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-500:], r.stderr[-1500:])
 
 
 def test_stream_probe_reports_a_plausible_rate_and_refuses_bad_sizes():
