@@ -48,6 +48,7 @@ struct GemmArgs {
     uint32_t c_prefetch;    // 1: beta != 0 and the old C may be fetched into freed LDS ring buffers ahead of the epilogue
     uint32_t c_stream;      // 1: C leaves with the non-temporal hint (x16 kernel; long k, many rounds of tiles)
     uint32_t line_rows;     // 1: A, B, their leading dimensions and batch strides are multiples of a 128-byte memory line
+    uint32_t ws_narrow;     // 1: a tile's span of the split-K workspace (tile columns x m floats) fits 32-bit offsets
 };
 
 // Linear work-group id -> (tile row, tile column).

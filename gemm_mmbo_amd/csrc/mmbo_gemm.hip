@@ -823,6 +823,7 @@ int gemm_impl(int dtype, int transA, int transB, size_t m, size_t n, size_t k,
         return ((uintptr_t)p % 128 == 0) && ((ld * esz) % 128 == 0) && (batch == 1 || ((size_t)stride * esz) % 128 == 0);
     };
     a.line_rows = on_lines(A, lda, strideA) && on_lines(B, ldb, strideB);
+    a.ws_narrow = (size_t)r.bn * m * 4 < 0x7FFFFF00ull;
     a.vec_c = aligned16(C, ldc, strideC) && (!cref.x16 || (size_t)r.bn * ldc * esz < 0x7FFFFF00ull);
     // beta != 0 on the x16 kernel's fp16 path: the old C of a tile is fetched into LDS under the tile's last slices (one
     // tile's span of C, tile columns x ldc, must then fit the 32-bit offsets of a buffer load)

@@ -32,7 +32,7 @@ constexpr TunedRow kTuned[] = {
     {0, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 52.2f},
     {1, 0, 0, 1023, 777, 513, 1, x16_id(4, 1), 89.9f},
     {0, 0, 0, 4096, 128, 4096, 1, ring_id(3, 4), 104.8f},
-    {1, 0, 0, 4096, 128, 4096, 1, ring_id(3, 2), 276.1f},
+    {1, 0, 0, 4096, 128, 4096, 1, x16_id(4, 2), 288.0f},
     {0, 0, 0, 128, 4096, 8192, 1, ring_id(1, 8), 118.9f},
     {1, 0, 0, 128, 4096, 8192, 1, ring_id(2, 4), 425.8f},
     {1, 1, 0, 512, 512, 512, 64, x16_id(0, 1), 650.0f},
